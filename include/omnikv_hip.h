@@ -1,0 +1,210 @@
+/*
+ * omnikv_hip.h - C ABI of libomnikv_hip.so: MI355X (gfx950) kernels for OmniKV's
+ * dynamic-context-selection decode path.
+ *
+ * The reference has no FFI layer of its own: the interface it exposes for this
+ * path is torch-level Python (modeling/omnikv.py, modeling/spec_cache.py) and,
+ * on its serving stack, Triton launchers.  Every entry point below names the
+ * reference code whose device work it replaces.  The Python package binds these
+ * with ctypes and re-creates the reference's Python signatures on top.
+ *
+ * Conventions
+ *   - plain pointers and sizes only; every pointer is a DEVICE pointer unless its
+ *     name starts with host_;
+ *   - every call is asynchronous on `stream` (a hipStream_t) and allocates
+ *     nothing: scratch comes from the caller as (ws, ws_bytes), sized by
+ *     okv_workspace_bytes();
+ *   - return value: 0 on success, a negative okv_status otherwise; the library
+ *     never throws and never aborts; okv_strerror() names a code and
+ *     okv_last_error() gives the detail of the calling thread's last failure;
+ *   - calls on different streams may run concurrently if their workspaces differ.
+ *
+ * Tensors
+ *   q, out     (batch, num_q_heads, head_dim) contiguous, same dtype as K/V
+ *   K, V       described by okv_kv_layout_t: element (b, t, g, d) of request b,
+ *              token t, kv head g lives at
+ *                contiguous: base + b*batch_stride + t*token_stride + g*head_stride + d
+ *                paged:      base + page_table[b*page_table_stride + t/page_size]*page_stride
+ *                                 + (t%page_size)*token_stride + g*head_stride + d
+ *              Both the reference's (b, Hkv, N, D) tensors (token_stride = D,
+ *              head_stride = N*D) and token-major (N, Hkv, D) storage
+ *              (token_stride = Hkv*D, head_stride = D) are expressible; strides
+ *              are in elements and must be multiples of 8; bases 16-byte aligned.
+ *   scores     (batch, score_stride) float32
+ *   idx        (batch, idx_stride) int32, ascending per request
+ */
+#ifndef OMNIKV_HIP_H
+#define OMNIKV_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* okv_stream_t; /* hipStream_t */
+
+enum okv_status {
+  OKV_OK = 0,
+  OKV_ERR_INVALID = -1,     /* bad argument (null pointer, misaligned, out of range) */
+  OKV_ERR_UNSUPPORTED = -2, /* geometry or dtype the kernels are not built for */
+  OKV_ERR_WORKSPACE = -3,   /* ws_bytes smaller than okv_workspace_bytes() */
+  OKV_ERR_HIP = -4          /* a HIP runtime call failed */
+};
+
+enum okv_dtype { OKV_F32 = 0, OKV_BF16 = 1, OKV_F16 = 2 };
+
+/* How the per-head logits of a token become one score. */
+enum okv_head_reduce { OKV_REDUCE_MAX = 0, OKV_REDUCE_SUM = 1 };
+enum okv_normalise { OKV_NORM_RAW = 0, OKV_NORM_SOFTMAX = 1 };
+
+enum okv_op {
+  OKV_OP_SCORE = 0,
+  OKV_OP_TOPK = 1,
+  OKV_OP_DENSE_ATTN = 2, /* with or without the fused score output */
+  OKV_OP_SPARSE_ATTN = 3
+};
+
+typedef struct okv_kv_layout {
+  int32_t dtype; /* okv_dtype */
+  int32_t num_q_heads;
+  int32_t num_kv_heads;
+  int32_t head_dim;
+  int64_t token_stride;
+  int64_t head_stride;
+  int64_t batch_stride;      /* contiguous mode only */
+  const int32_t* page_table; /* device; NULL selects contiguous mode */
+  int32_t page_size;
+  int32_t page_table_stride; /* entries per request */
+  int64_t page_stride;
+} okv_kv_layout_t;
+
+/* Sizes that determine a workspace: fill what the op uses, zero the rest. */
+typedef struct okv_shape {
+  int32_t batch;
+  int32_t num_q_heads;
+  int32_t num_kv_heads;
+  int32_t head_dim;
+  int32_t max_seq_len;  /* longest scored / attended main segment */
+  int32_t max_tail_len; /* sparse attention only */
+  int32_t with_scores;  /* dense attention: 1 when the score output is wanted */
+} okv_shape_t;
+
+const char* okv_strerror(int status);
+const char* okv_last_error(void);
+int okv_version(void);
+
+/* Bytes of scratch `op` needs for `shape`.  No reference counterpart: the
+ * reference lets torch allocate (alloc_tensor_func in
+ * omnikv-lightllm/.../triton_kernel/flash_decoding.py:45-60). */
+int okv_workspace_bytes(int op, const okv_shape_t* shape, size_t* out_bytes);
+
+/*
+ * Filter-layer scoring.  For each request b and token t < score_len:
+ *   logit[h][t] = scale * <q[b][h], K[b][t][h / group]>
+ *   RAW:      s[h][t] = logit[h][t]
+ *   SOFTMAX:  s[h][t] = softmax over t in [0, score_len) of logit[h][.]
+ *   scores[b][t] = max_h or sum_h of s[h][t]
+ * Replaces the matmul / softmax / max chain of select_tokens_by_attn_universal,
+ * branches `last` (RAW+MAX) and `softmax_before_last` (SOFTMAX+MAX):
+ * modeling/omnikv.py:37-58; and the raw-score side output of
+ * _fwd_kernel_flash_decode_stage1_with_score + attn_score.max(dim=1):
+ * omnikv-lightllm/.../flash_decoding_stage1.py:198-207, flash_decoding.py:76.
+ * score_lens: device int32[batch] or NULL (then every request has max_score_len).
+ */
+int okv_score(const void* q, const void* k_base, const okv_kv_layout_t* layout,
+              const int32_t* score_lens, int32_t max_score_len, int32_t batch,
+              int32_t head_reduce, int32_t normalise, float scale, float* scores,
+              int64_t score_stride, void* ws, size_t ws_bytes, okv_stream_t stream);
+
+/*
+ * Per-request top-k of fp32 scores.  Writes the k_b = min(k_per_seg[b], len_b)
+ * selected token indices in ASCENDING order.  The selected set holds every value
+ * greater than the k-th largest and, among values equal to it, those with the
+ * lowest indices.  -0.0 equals +0.0; NaN ranks above +inf.
+ * Replaces torch.topk(sorted=True) followed by torch.sort(idx):
+ * modeling/omnikv.py:47-48,109; and torch.topk in
+ * omnikv-lightllm/.../flash_decoding.py:80-83.
+ * seq_lens / k_per_seg: device int32[batch] or NULL (then max_seq_len / max_k
+ * apply to every request).  idx_out rows beyond k_b are left untouched.
+ */
+int okv_topk(const float* scores, int64_t score_stride, const int32_t* seq_lens,
+             int32_t max_seq_len, const int32_t* k_per_seg, int32_t max_k,
+             int32_t batch, int32_t* idx_out, int64_t idx_stride, void* ws,
+             size_t ws_bytes, okv_stream_t stream);
+
+/*
+ * Dense GQA decode attention over all seq_len cached tokens of each request:
+ * out[b][h] = softmax_t(scale * <q[b][h], K[b][t][h/group]>) . V[b][.][h/group].
+ * When `scores` is not NULL the same pass over K also emits the filter-layer
+ * scores of the first score_len tokens, exactly as okv_score would (the softmax
+ * of the score is over [0, score_len), that of the attention over [0, seq_len)).
+ * Replaces the attention the reference runs on a full layer after
+ * OmniKVMultiStageCache.update returns the whole cache
+ * (modeling/spec_cache.py:358-369, called from modeling/omnikv.py:219-227) and
+ * flash_decode_stage1(_with_score) + flash_decode_stage2
+ * (omnikv-lightllm/.../flash_decoding.py:62-75,107-112).
+ */
+int okv_dense_attn(const void* q, const void* k_base, const void* v_base,
+                   const okv_kv_layout_t* layout, const int32_t* seq_lens,
+                   int32_t max_seq_len, int32_t batch, float scale, void* out,
+                   const int32_t* score_lens, int32_t max_score_len,
+                   int32_t head_reduce, int32_t normalise, float* scores,
+                   int64_t score_stride, void* ws, size_t ws_bytes,
+                   okv_stream_t stream);
+
+/*
+ * Fused gather + sparse GQA decode attention.  Request b attends to the rows
+ *   K/V[b][idx[b][0 .. sel_len_b)]  followed by  tail_K/V[b][0 .. tail_len_b)
+ * with one joint softmax.  idx == NULL means rows 0 .. sel_len_b-1 of K/V (an
+ * already gathered buffer).  The tail (tokens generated after the prompt) is
+ * (batch, tail_len, Hkv, D)-addressed by its own three strides; tail_k may be
+ * NULL when max_tail_len == 0.
+ * Replaces index_select in set_idx_on_gpu, torch.cat([part, tail]) in update,
+ * and the attention over the result: modeling/spec_cache.py:290-306,337-356,
+ * modeling/omnikv.py:219-227; and flash_decode_stage1 over
+ * req_to_imp_token_indexs: omnikv-lightllm/.../flash_decoding.py:93-105.
+ */
+int okv_sparse_attn(const void* q, const void* k_base, const void* v_base,
+                    const okv_kv_layout_t* layout, const int32_t* idx,
+                    int64_t idx_stride, const int32_t* sel_lens, int32_t max_sel_len,
+                    const void* tail_k, const void* tail_v, int64_t tail_token_stride,
+                    int64_t tail_head_stride, int64_t tail_batch_stride,
+                    const int32_t* tail_lens, int32_t max_tail_len, int32_t batch,
+                    float scale, void* out, void* ws, size_t ws_bytes,
+                    okv_stream_t stream);
+
+/*
+ * Materialised gather: dst[b][j][g][:] = src[b][idx[b][j]][g][:] for j < sel_len_b,
+ * dst addressed by (dst_token_stride, dst_head_stride, dst_batch_stride).
+ * Replaces torch.index_select(cache, 2, idx) in set_idx_on_gpu
+ * (modeling/spec_cache.py:298-303) for callers that need the gathered tensor
+ * itself (a third-party attention consuming update()'s return value).
+ */
+int okv_gather_rows(const void* src_base, const okv_kv_layout_t* layout,
+                    const int32_t* idx, int64_t idx_stride, const int32_t* sel_lens,
+                    int32_t max_sel_len, int32_t batch, void* dst,
+                    int64_t dst_token_stride, int64_t dst_head_stride,
+                    int64_t dst_batch_stride, okv_stream_t stream);
+
+/*
+ * real_offload tier.  Copies the selected rows of one layer's K and V from PINNED
+ * host memory (token-major rows of row_bytes bytes, row t at host_src + t*row_bytes)
+ * into a contiguous device buffer, asynchronously on copy_stream, and records
+ * done_event (a hipEvent_t, may be NULL) behind the copy.  host_idx is a HOST
+ * array of n_rows ascending token indices.  Rows are packed by host_threads
+ * CPU threads (>= 1; the call returns when packing is done) into host_staging
+ * (pinned, >= n_rows*row_bytes) and moved with one hipMemcpyAsync.  The caller
+ * must not reuse host_staging before done_event has completed.
+ * Replaces `index_select(cpu cache, 2, idx.cpu()).cuda(non_blocking=True)`:
+ * modeling/spec_cache.py:293-303.
+ */
+int okv_offload_stage(const void* host_src, int64_t row_bytes, const int32_t* host_idx,
+                      int32_t n_rows, void* host_staging, int32_t host_threads,
+                      void* dev_dst, okv_stream_t copy_stream, void* done_event);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OMNIKV_HIP_H */

@@ -1,0 +1,113 @@
+"""ctypes binding of libomnikv_hip.so (declared in include/omnikv_hip.h).
+
+The library is required: there is no CPU or torch fallback.  `lib()` raises
+OmniKVLibraryError when the shared object has not been built, and every wrapper
+turns a negative status into an exception carrying okv_last_error().
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libomnikv_hip.so")
+
+OKV_F32, OKV_BF16, OKV_F16 = 0, 1, 2
+OKV_REDUCE_MAX, OKV_REDUCE_SUM = 0, 1
+OKV_NORM_RAW, OKV_NORM_SOFTMAX = 0, 1
+OKV_OP_SCORE, OKV_OP_TOPK, OKV_OP_DENSE_ATTN, OKV_OP_SPARSE_ATTN = 0, 1, 2, 3
+
+EXPORTS = (
+    "okv_strerror",
+    "okv_last_error",
+    "okv_version",
+    "okv_workspace_bytes",
+    "okv_score",
+    "okv_topk",
+    "okv_dense_attn",
+    "okv_sparse_attn",
+    "okv_gather_rows",
+    "okv_offload_stage",
+)
+
+
+class OmniKVLibraryError(RuntimeError):
+    pass
+
+
+class KVLayout(C.Structure):
+    _fields_ = [
+        ("dtype", C.c_int32),
+        ("num_q_heads", C.c_int32),
+        ("num_kv_heads", C.c_int32),
+        ("head_dim", C.c_int32),
+        ("token_stride", C.c_int64),
+        ("head_stride", C.c_int64),
+        ("batch_stride", C.c_int64),
+        ("page_table", C.c_void_p),
+        ("page_size", C.c_int32),
+        ("page_table_stride", C.c_int32),
+        ("page_stride", C.c_int64),
+    ]
+
+
+class Shape(C.Structure):
+    _fields_ = [
+        ("batch", C.c_int32),
+        ("num_q_heads", C.c_int32),
+        ("num_kv_heads", C.c_int32),
+        ("head_dim", C.c_int32),
+        ("max_seq_len", C.c_int32),
+        ("max_tail_len", C.c_int32),
+        ("with_scores", C.c_int32),
+    ]
+
+
+_lib = None
+
+
+def _declare(l):
+    vp, i32, i64, f32, sz = C.c_void_p, C.c_int32, C.c_int64, C.c_float, C.c_size_t
+    l.okv_strerror.restype = C.c_char_p
+    l.okv_strerror.argtypes = [C.c_int]
+    l.okv_last_error.restype = C.c_char_p
+    l.okv_last_error.argtypes = []
+    l.okv_version.restype = C.c_int
+    l.okv_version.argtypes = []
+    l.okv_workspace_bytes.restype = C.c_int
+    l.okv_workspace_bytes.argtypes = [C.c_int, C.POINTER(Shape), C.POINTER(sz)]
+    l.okv_score.restype = C.c_int
+    l.okv_score.argtypes = [vp, vp, C.POINTER(KVLayout), vp, i32, i32, i32, i32, f32, vp, i64, vp, sz, vp]
+    l.okv_topk.restype = C.c_int
+    l.okv_topk.argtypes = [vp, i64, vp, i32, vp, i32, i32, vp, i64, vp, sz, vp]
+    l.okv_dense_attn.restype = C.c_int
+    l.okv_dense_attn.argtypes = [vp, vp, vp, C.POINTER(KVLayout), vp, i32, i32, f32, vp, vp, i32, i32, i32, vp, i64, vp, sz, vp]
+    l.okv_sparse_attn.restype = C.c_int
+    l.okv_sparse_attn.argtypes = [vp, vp, vp, C.POINTER(KVLayout), vp, i64, vp, i32, vp, vp, i64, i64, i64, vp, i32, i32, f32, vp, vp, sz, vp]
+    l.okv_gather_rows.restype = C.c_int
+    l.okv_gather_rows.argtypes = [vp, C.POINTER(KVLayout), vp, i64, vp, i32, i32, vp, i64, i64, i64, vp]
+    l.okv_offload_stage.restype = C.c_int
+    l.okv_offload_stage.argtypes = [vp, i64, vp, i32, vp, i32, vp, vp, vp]
+
+
+def lib():
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise OmniKVLibraryError(
+                f"{LIB_PATH} is missing: build it with `python omnikv_amd/csrc/build.py` "
+                "(hipcc, gfx950). There is no fallback path."
+            )
+        l = C.CDLL(LIB_PATH)
+        _declare(l)
+        _lib = l
+    return _lib
+
+
+def check(status: int) -> None:
+    if status != 0:
+        l = lib()
+        raise OmniKVLibraryError(
+            f"{l.okv_strerror(status).decode()} ({status}): {l.okv_last_error().decode()}"
+        )

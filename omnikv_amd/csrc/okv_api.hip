@@ -1,0 +1,156 @@
+// Status strings, argument validation and workspace sizing of libomnikv_hip.so.
+#include <stdarg.h>
+#include <string.h>
+
+#include "okv_internal.h"
+
+namespace okv {
+
+static thread_local char g_last_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+  va_end(ap);
+}
+
+static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// Rows per split: enough blocks to fill 256 CUs several times over for long
+// contexts, never below one 64-row tile group.
+static int choose_split_rows(int batch, int hkv, int total_rows) {
+  const int64_t target_blocks = 4096;
+  int64_t work = (int64_t)total_rows * hkv * (batch > 0 ? batch : 1);
+  int64_t rows = (work + target_blocks - 1) / target_blocks;
+  rows = (rows + 63) / 64 * 64;
+  if (rows < 64) rows = 64;
+  if (rows > 1024) rows = 1024;
+  return (int)rows;
+}
+
+size_t attn_workspace_bytes(int batch, int hq, int hkv, int d, int max_main, int max_tail,
+                            int max_score, bool with_v, bool with_logits, int* split_rows,
+                            int* max_splits) {
+  int L = max_main + max_tail;
+  int C = choose_split_rows(batch, hkv, L);
+  int S = (L + C - 1) / C + (max_score > 0 ? 1 : 0);
+  if (S < 1) S = 1;
+  if (split_rows) *split_rows = C;
+  if (max_splits) *max_splits = S;
+  size_t bytes = 0;
+  if (with_v) bytes += align_up((size_t)batch * hq * S * d * sizeof(float), 256);
+  bytes += align_up((size_t)batch * hq * S * sizeof(float), 256);
+  if (with_logits) {
+    size_t ls = align_up((size_t)max_score, 64);
+    bytes += align_up((size_t)batch * hq * ls * sizeof(float), 256);
+  }
+  bytes += align_up((size_t)batch * hq * sizeof(float), 256);
+  return bytes + 256;
+}
+
+int carve_attn_workspace(void* ws, size_t ws_bytes, int batch, int hq, int hkv, int d,
+                         int max_main, int max_tail, int max_score, bool with_v,
+                         bool with_logits, AttnWorkspace* out) {
+  int C = 0, S = 0;
+  size_t need = attn_workspace_bytes(batch, hq, hkv, d, max_main, max_tail, max_score, with_v,
+                                     with_logits, &C, &S);
+  OKV_REQUIRE(ws != nullptr, OKV_ERR_INVALID, "workspace pointer is NULL");
+  OKV_REQUIRE(ws_bytes >= need, OKV_ERR_WORKSPACE, "workspace too small: have %zu, need %zu",
+              ws_bytes, need);
+  char* p = (char*)align_up((size_t)ws, 256);
+  memset(out, 0, sizeof(*out));
+  out->split_rows = C;
+  out->max_splits = S;
+  if (with_v) {
+    out->part_o = (float*)p;
+    p += align_up((size_t)batch * hq * S * d * sizeof(float), 256);
+  }
+  out->part_lse = (float*)p;
+  p += align_up((size_t)batch * hq * S * sizeof(float), 256);
+  if (with_logits) {
+    out->logits_stride = (int64_t)align_up((size_t)max_score, 64);
+    out->logits = (float*)p;
+    p += align_up((size_t)batch * hq * out->logits_stride * sizeof(float), 256);
+  }
+  out->score_lse = (float*)p;
+  return OKV_OK;
+}
+
+int validate_layout(const okv_kv_layout_t* layout, const void* k_base, const void* v_base) {
+  OKV_REQUIRE(layout != nullptr, OKV_ERR_INVALID, "layout is NULL");
+  OKV_REQUIRE(k_base != nullptr, OKV_ERR_INVALID, "k_base is NULL");
+  OKV_REQUIRE(layout->dtype == OKV_F32 || layout->dtype == OKV_BF16 || layout->dtype == OKV_F16,
+              OKV_ERR_UNSUPPORTED, "dtype %d not supported", layout->dtype);
+  OKV_REQUIRE(layout->head_dim == 128, OKV_ERR_UNSUPPORTED,
+              "head_dim %d not supported (kernels are built for 128)", layout->head_dim);
+  OKV_REQUIRE(layout->num_kv_heads >= 1 && layout->num_q_heads >= layout->num_kv_heads &&
+                  layout->num_q_heads % layout->num_kv_heads == 0,
+              OKV_ERR_INVALID, "bad head counts q=%d kv=%d", layout->num_q_heads,
+              layout->num_kv_heads);
+  int group = layout->num_q_heads / layout->num_kv_heads;
+  OKV_REQUIRE(group == 1 || group == 2 || group == 4 || group == 8, OKV_ERR_UNSUPPORTED,
+              "GQA group size %d not supported (1, 2, 4, 8)", group);
+  OKV_REQUIRE(layout->token_stride % 8 == 0 && layout->head_stride % 8 == 0 &&
+                  layout->batch_stride % 8 == 0 && layout->page_stride % 8 == 0,
+              OKV_ERR_INVALID, "strides must be multiples of 8 elements");
+  OKV_REQUIRE(((uintptr_t)k_base & 15) == 0 && ((uintptr_t)v_base & 15) == 0, OKV_ERR_INVALID,
+              "K/V base pointers must be 16-byte aligned");
+  if (layout->page_table) {
+    OKV_REQUIRE(layout->page_size >= 1, OKV_ERR_INVALID, "page_size must be >= 1");
+    OKV_REQUIRE(layout->page_table_stride >= 1, OKV_ERR_INVALID, "page_table_stride must be >= 1");
+  }
+  return OKV_OK;
+}
+
+}  // namespace okv
+
+extern "C" {
+
+const char* okv_strerror(int status) {
+  switch (status) {
+    case OKV_OK: return "ok";
+    case OKV_ERR_INVALID: return "invalid argument";
+    case OKV_ERR_UNSUPPORTED: return "unsupported geometry or dtype";
+    case OKV_ERR_WORKSPACE: return "workspace too small";
+    case OKV_ERR_HIP: return "HIP runtime error";
+    default: return "unknown status";
+  }
+}
+
+const char* okv_last_error(void) { return okv::g_last_error; }
+
+int okv_version(void) { return 1; }
+
+int okv_workspace_bytes(int op, const okv_shape_t* s, size_t* out_bytes) {
+  OKV_REQUIRE(s != nullptr && out_bytes != nullptr, OKV_ERR_INVALID, "NULL argument");
+  OKV_REQUIRE(s->batch >= 1, OKV_ERR_INVALID, "batch must be >= 1");
+  OKV_REQUIRE(op == OKV_OP_TOPK || (s->num_q_heads >= 1 && s->num_kv_heads >= 1 && s->head_dim >= 1),
+              OKV_ERR_INVALID, "head counts and head_dim must be >= 1");
+  switch (op) {
+    case OKV_OP_SCORE:
+      *out_bytes = okv::attn_workspace_bytes(s->batch, s->num_q_heads, s->num_kv_heads, s->head_dim,
+                                             s->max_seq_len, 0, s->max_seq_len, false, true,
+                                             nullptr, nullptr);
+      return OKV_OK;
+    case OKV_OP_DENSE_ATTN:
+      *out_bytes = okv::attn_workspace_bytes(s->batch, s->num_q_heads, s->num_kv_heads, s->head_dim,
+                                             s->max_seq_len, 0,
+                                             s->with_scores ? s->max_seq_len : 0, true,
+                                             s->with_scores != 0, nullptr, nullptr);
+      return OKV_OK;
+    case OKV_OP_SPARSE_ATTN:
+      *out_bytes = okv::attn_workspace_bytes(s->batch, s->num_q_heads, s->num_kv_heads, s->head_dim,
+                                             s->max_seq_len, s->max_tail_len, 0, true, false,
+                                             nullptr, nullptr);
+      return OKV_OK;
+    case OKV_OP_TOPK:
+      *out_bytes = 256;  // the selector keeps its state in LDS
+      return OKV_OK;
+    default:
+      okv::set_error("unknown op %d", op);
+      return OKV_ERR_INVALID;
+  }
+}
+
+}  // extern "C"

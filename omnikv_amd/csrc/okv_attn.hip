@@ -1,0 +1,434 @@
+// Split-context GQA decode attention and filter-layer scoring for gfx950.
+//
+// One pass over the rows of a request (stage 1) produces, per (q head, split),
+// a normalised partial output and its log-sum-exp, and optionally the scaled
+// logits of the scored rows.  A merge kernel combines the splits; a finishing
+// kernel turns logits into one score per token.
+//
+// This file holds the portable wave64 VALU formulation (any of f32 / bf16 / f16,
+// GQA group 1..8): sixteen lanes share a 128-element row, eight elements each.
+#include <math.h>
+#include <string.h>
+
+#include "okv_internal.h"
+
+namespace okv {
+
+static constexpr float kLog2e = 1.4426950408889634f;
+static constexpr int kD = 128;
+
+struct BF16 {
+  uint16_t v;
+};
+struct F16 {
+  uint16_t v;
+};
+
+// ---- eight consecutive elements -> fp32
+__device__ __forceinline__ void load8(const float* p, float* o) {
+  float4 a = *reinterpret_cast<const float4*>(p);
+  float4 b = *reinterpret_cast<const float4*>(p + 4);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+  o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+__device__ __forceinline__ void load8(const BF16* p, float* o) {
+  uint4 u = *reinterpret_cast<const uint4*>(p);
+  o[0] = __uint_as_float(u.x << 16); o[1] = __uint_as_float(u.x & 0xffff0000u);
+  o[2] = __uint_as_float(u.y << 16); o[3] = __uint_as_float(u.y & 0xffff0000u);
+  o[4] = __uint_as_float(u.z << 16); o[5] = __uint_as_float(u.z & 0xffff0000u);
+  o[6] = __uint_as_float(u.w << 16); o[7] = __uint_as_float(u.w & 0xffff0000u);
+}
+__device__ __forceinline__ void load8(const F16* p, float* o) {
+  uint4 u = *reinterpret_cast<const uint4*>(p);
+  const _Float16* h = reinterpret_cast<const _Float16*>(&u);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = (float)h[i];
+}
+
+__device__ __forceinline__ void store1(float* p, float v) { *p = v; }
+__device__ __forceinline__ void store1(BF16* p, float v) {
+  uint32_t u = __float_as_uint(v);
+  uint16_t r;
+  if ((u & 0x7fffffffu) > 0x7f800000u) {
+    r = 0x7fc0;  // NaN
+  } else {
+    u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
+    r = (uint16_t)(u >> 16);
+  }
+  p->v = r;
+}
+__device__ __forceinline__ void store1(F16* p, float v) {
+  _Float16 h = (_Float16)v;
+  p->v = *reinterpret_cast<uint16_t*>(&h);
+}
+
+// ----------------------------------------------------------------- stage 1
+// grid (splits, kv heads, batch), 256 threads.  Each group of 16 lanes walks
+// every 16th row of the split, keeping a private online-softmax state for the G
+// q heads of the kv head; the 16 groups of the block are merged at the end.
+template <typename T, int G, bool WITH_V>
+__global__ __launch_bounds__(256) void attn_stage1_generic(const T* __restrict__ q, RowList rows,
+                                                           int hq, float scale, AttnWorkspace w,
+                                                           int write_logits) {
+  const int split = blockIdx.x, g = blockIdx.y, b = blockIdx.z;
+  const int main_len = rl_main_len(rows, b);
+  const int L = main_len + rl_tail_len(rows, b);
+  const int A = rl_score_len(rows, b);
+  int begin, end;
+  rl_split_range(split, w.split_rows, A, L, &begin, &end);
+  if (begin >= end) return;
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = lane & 15;
+  const int grp = wave * 4 + (lane >> 4);
+
+  float qr[G][8];
+#pragma unroll
+  for (int h = 0; h < G; ++h) load8(q + ((int64_t)(b * hq + g * G + h) * kD + c * 8), qr[h]);
+
+  float m[G], l[G], acc[G][8];
+#pragma unroll
+  for (int h = 0; h < G; ++h) {
+    m[h] = -INFINITY;
+    l[h] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
+  }
+  const float sl2 = scale * kLog2e;
+  const T* kb = reinterpret_cast<const T*>(rows.k_base);
+  const T* vb = reinterpret_cast<const T*>(rows.v_base);
+  const T* tkb = reinterpret_cast<const T*>(rows.tail_k);
+  const T* tvb = reinterpret_cast<const T*>(rows.tail_v);
+
+  for (int row = begin + grp; row < end; row += 16) {
+    bool in_tail;
+    int64_t off = rl_row_offset(rows, b, row, main_len, &in_tail);
+    off += (int64_t)g * (in_tail ? rows.tail_head_stride : rows.head_stride) + c * 8;
+    float kf[8];
+    load8((in_tail ? tkb : kb) + off, kf);
+    float s[G];
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      float a = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) a = fmaf(qr[h][i], kf[i], a);
+      a += __shfl_xor(a, 8);
+      a += __shfl_xor(a, 4);
+      a += __shfl_xor(a, 2);
+      a += __shfl_xor(a, 1);
+      s[h] = a;
+    }
+    if (write_logits && row < A) {
+#pragma unroll
+      for (int h = 0; h < G; ++h)
+        if (c == h) w.logits[(int64_t)(b * hq + g * G + h) * w.logits_stride + row] = s[h] * scale;
+    }
+    float vf[8];
+    if (WITH_V) load8((in_tail ? tvb : vb) + off, vf);
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      float s2 = s[h] * sl2;
+      float mn = fmaxf(m[h], s2);
+      float alpha = exp2f(m[h] - mn);
+      float p = exp2f(s2 - mn);
+      l[h] = l[h] * alpha + p;
+      m[h] = mn;
+      if (WITH_V) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[h][i] = acc[h][i] * alpha + p * vf[i];
+      }
+    }
+  }
+
+  // merge the four 16-lane groups of the wave (lanes l, l^16, l^32, l^48)
+#pragma unroll
+  for (int h = 0; h < G; ++h) {
+    float M = fmaxf(m[h], __shfl_xor(m[h], 16));
+    M = fmaxf(M, __shfl_xor(M, 32));
+    float f = (m[h] == -INFINITY) ? 0.f : exp2f(m[h] - M);
+    float ll = l[h] * f;
+    ll += __shfl_xor(ll, 16);
+    ll += __shfl_xor(ll, 32);
+    l[h] = ll;
+    m[h] = M;
+    if (WITH_V) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float a = acc[h][i] * f;
+        a += __shfl_xor(a, 16);
+        a += __shfl_xor(a, 32);
+        acc[h][i] = a;
+      }
+    }
+  }
+
+  __shared__ float sm[4][G];
+  __shared__ float sl[4][G];
+  __shared__ float sacc[WITH_V ? 4 : 1][G][kD];
+  if (lane < 16) {
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      if (c == 0) {
+        sm[wave][h] = m[h];
+        sl[wave][h] = l[h];
+      }
+      if (WITH_V) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sacc[wave][h][c * 8 + i] = acc[h][i];
+      }
+    }
+  }
+  __syncthreads();
+  for (int o = threadIdx.x; o < G * kD; o += 256) {
+    const int h = o / kD, d = o % kD;
+    float M = fmaxf(fmaxf(sm[0][h], sm[1][h]), fmaxf(sm[2][h], sm[3][h]));
+    float den = 0.f, num = 0.f;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      float f = (sm[x][h] == -INFINITY) ? 0.f : exp2f(sm[x][h] - M);
+      den += sl[x][h] * f;
+      if (WITH_V) num += sacc[x][h][d] * f;
+    }
+    const int64_t ph = (int64_t)(b * hq + g * G + h) * w.max_splits + split;
+    if (WITH_V) w.part_o[ph * kD + d] = num / den;
+    if (d == 0) w.part_lse[ph] = M + log2f(den);
+  }
+}
+
+// ------------------------------------------------------------------- merge
+// grid (q heads, batch), 128 threads (one per output element).
+template <typename T>
+__global__ __launch_bounds__(128) void attn_merge(RowList rows, int hq, AttnWorkspace w,
+                                                  T* __restrict__ out, int with_v,
+                                                  int with_score_lse) {
+  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  const int main_len = rl_main_len(rows, b);
+  const int L = main_len + rl_tail_len(rows, b);
+  const int A = rl_score_len(rows, b);
+  const int ns = rl_num_splits(w.split_rows, A, L);
+  const int nA = (A + w.split_rows - 1) / w.split_rows;
+  const int64_t ph = (int64_t)(b * hq + h) * w.max_splits;
+  if (with_v) {
+    float M = -INFINITY;
+    for (int s = 0; s < ns; ++s) M = fmaxf(M, w.part_lse[ph + s]);
+    float den = 0.f, num = 0.f;
+    for (int s = 0; s < ns; ++s) {
+      float f = exp2f(w.part_lse[ph + s] - M);
+      den += f;
+      num += f * w.part_o[(ph + s) * kD + d];
+    }
+    store1(out + (int64_t)(b * hq + h) * kD + d, ns > 0 ? num / den : 0.f);
+  }
+  if (with_score_lse && d == 0) {
+    float M = -INFINITY;
+    for (int s = 0; s < nA; ++s) M = fmaxf(M, w.part_lse[ph + s]);
+    float den = 0.f;
+    for (int s = 0; s < nA; ++s) den += exp2f(w.part_lse[ph + s] - M);
+    w.score_lse[b * hq + h] = M + log2f(den);
+  }
+}
+
+// ------------------------------------------------------------ score finish
+// grid (ceil(max_score/256), batch), 256 threads, one token each.
+__global__ __launch_bounds__(256) void score_finish(RowList rows, int hq, AttnWorkspace w,
+                                                    int head_reduce, int normalise,
+                                                    float* __restrict__ scores,
+                                                    int64_t score_stride) {
+  const int b = blockIdx.y;
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  const int A = rl_score_len(rows, b);
+  if (t >= A) return;
+  float acc = head_reduce == OKV_REDUCE_MAX ? -INFINITY : 0.f;
+  for (int h = 0; h < hq; ++h) {
+    float v = w.logits[(int64_t)(b * hq + h) * w.logits_stride + t];
+    if (normalise == OKV_NORM_SOFTMAX) v = exp2f(v * kLog2e - w.score_lse[b * hq + h]);
+    acc = head_reduce == OKV_REDUCE_MAX ? fmaxf(acc, v) : acc + v;
+  }
+  scores[(int64_t)b * score_stride + t] = acc;
+}
+
+// ----------------------------------------------------------------- launch
+template <typename T, int G>
+static void launch_stage1(const void* q, const RowList& rows, int hq, int hkv, int batch,
+                          float scale, const AttnWorkspace& w, bool with_v, bool write_logits,
+                          hipStream_t stream) {
+  dim3 grid(w.max_splits, hkv, batch);
+  if (with_v)
+    hipLaunchKernelGGL((attn_stage1_generic<T, G, true>), grid, dim3(256), 0, stream,
+                       (const T*)q, rows, hq, scale, w, (int)write_logits);
+  else
+    hipLaunchKernelGGL((attn_stage1_generic<T, G, false>), grid, dim3(256), 0, stream,
+                       (const T*)q, rows, hq, scale, w, (int)write_logits);
+}
+
+template <typename T>
+static int launch_typed(const void* q, const RowList& rows, const okv_kv_layout_t* lay,
+                        int batch, float scale, void* out, bool with_v, int head_reduce,
+                        int normalise, float* scores, int64_t score_stride,
+                        const AttnWorkspace& w, hipStream_t stream) {
+  const int hq = lay->num_q_heads, hkv = lay->num_kv_heads, G = hq / hkv;
+  const bool want_scores = scores != nullptr;
+  switch (G) {
+    case 1: launch_stage1<T, 1>(q, rows, hq, hkv, batch, scale, w, with_v, want_scores, stream); break;
+    case 2: launch_stage1<T, 2>(q, rows, hq, hkv, batch, scale, w, with_v, want_scores, stream); break;
+    case 4: launch_stage1<T, 4>(q, rows, hq, hkv, batch, scale, w, with_v, want_scores, stream); break;
+    case 8: launch_stage1<T, 8>(q, rows, hq, hkv, batch, scale, w, with_v, want_scores, stream); break;
+    default: set_error("GQA group %d not supported", G); return OKV_ERR_UNSUPPORTED;
+  }
+  const bool need_score_lse = want_scores && normalise == OKV_NORM_SOFTMAX;
+  if (with_v || need_score_lse)
+    hipLaunchKernelGGL((attn_merge<T>), dim3(hq, batch), dim3(128), 0, stream, rows, hq, w,
+                       (T*)out, (int)with_v, (int)need_score_lse);
+  if (want_scores && rows.max_score_len > 0)
+    hipLaunchKernelGGL(score_finish, dim3((rows.max_score_len + 255) / 256, batch), dim3(256), 0,
+                       stream, rows, hq, w, head_reduce, normalise, scores, score_stride);
+  OKV_HIP_CHECK(hipGetLastError());
+  return OKV_OK;
+}
+
+int launch_attention(const void* q, const RowList& rows, const okv_kv_layout_t* lay, int batch,
+                     float scale, void* out, bool with_v, int head_reduce, int normalise,
+                     float* scores, int64_t score_stride, const AttnWorkspace& w,
+                     hipStream_t stream) {
+  switch (lay->dtype) {
+    case OKV_F32:
+      return launch_typed<float>(q, rows, lay, batch, scale, out, with_v, head_reduce, normalise,
+                                 scores, score_stride, w, stream);
+    case OKV_BF16:
+      return launch_typed<BF16>(q, rows, lay, batch, scale, out, with_v, head_reduce, normalise,
+                                scores, score_stride, w, stream);
+    case OKV_F16:
+      return launch_typed<F16>(q, rows, lay, batch, scale, out, with_v, head_reduce, normalise,
+                               scores, score_stride, w, stream);
+  }
+  set_error("dtype %d not supported", lay->dtype);
+  return OKV_ERR_UNSUPPORTED;
+}
+
+static void fill_main(RowList* r, const void* k, const void* v, const okv_kv_layout_t* lay) {
+  memset(r, 0, sizeof(*r));
+  r->k_base = k;
+  r->v_base = v;
+  r->token_stride = lay->token_stride;
+  r->head_stride = lay->head_stride;
+  r->batch_stride = lay->batch_stride;
+  r->page_table = lay->page_table;
+  r->page_size = lay->page_size;
+  r->page_table_stride = lay->page_table_stride;
+  r->page_stride = lay->page_stride;
+}
+
+}  // namespace okv
+
+using namespace okv;
+
+extern "C" {
+
+int okv_score(const void* q, const void* k_base, const okv_kv_layout_t* layout,
+              const int32_t* score_lens, int32_t max_score_len, int32_t batch,
+              int32_t head_reduce, int32_t normalise, float scale, float* scores,
+              int64_t score_stride, void* ws, size_t ws_bytes, okv_stream_t stream) {
+  int rc = validate_layout(layout, k_base, k_base);
+  if (rc) return rc;
+  OKV_REQUIRE(q && scores, OKV_ERR_INVALID, "q or scores is NULL");
+  OKV_REQUIRE(batch >= 1 && max_score_len >= 0, OKV_ERR_INVALID, "bad batch or length");
+  OKV_REQUIRE(score_stride >= max_score_len, OKV_ERR_INVALID, "score_stride < max_score_len");
+  OKV_REQUIRE(head_reduce == OKV_REDUCE_MAX || head_reduce == OKV_REDUCE_SUM, OKV_ERR_INVALID,
+              "bad head_reduce %d", head_reduce);
+  OKV_REQUIRE(normalise == OKV_NORM_RAW || normalise == OKV_NORM_SOFTMAX, OKV_ERR_INVALID,
+              "bad normalise %d", normalise);
+  if (max_score_len == 0) return OKV_OK;
+  AttnWorkspace w;
+  rc = carve_attn_workspace(ws, ws_bytes, batch, layout->num_q_heads, layout->num_kv_heads,
+                            layout->head_dim, max_score_len, 0, max_score_len, false, true, &w);
+  if (rc) return rc;
+  RowList r;
+  fill_main(&r, k_base, k_base, layout);
+  r.main_lens = score_lens;
+  r.max_main_len = max_score_len;
+  r.score_lens = score_lens;
+  r.max_score_len = max_score_len;
+  return launch_attention(q, r, layout, batch, scale, nullptr, false, head_reduce, normalise,
+                          scores, score_stride, w, (hipStream_t)stream);
+}
+
+int okv_dense_attn(const void* q, const void* k_base, const void* v_base,
+                   const okv_kv_layout_t* layout, const int32_t* seq_lens, int32_t max_seq_len,
+                   int32_t batch, float scale, void* out, const int32_t* score_lens,
+                   int32_t max_score_len, int32_t head_reduce, int32_t normalise, float* scores,
+                   int64_t score_stride, void* ws, size_t ws_bytes, okv_stream_t stream) {
+  int rc = validate_layout(layout, k_base, v_base);
+  if (rc) return rc;
+  OKV_REQUIRE(q && out && v_base, OKV_ERR_INVALID, "q, v_base or out is NULL");
+  OKV_REQUIRE(batch >= 1 && max_seq_len >= 1, OKV_ERR_INVALID, "bad batch or length");
+  if (scores) {
+    OKV_REQUIRE(max_score_len >= 0 && max_score_len <= max_seq_len, OKV_ERR_INVALID,
+                "max_score_len out of range");
+    OKV_REQUIRE(score_stride >= max_score_len, OKV_ERR_INVALID, "score_stride < max_score_len");
+    OKV_REQUIRE(head_reduce == OKV_REDUCE_MAX || head_reduce == OKV_REDUCE_SUM, OKV_ERR_INVALID,
+                "bad head_reduce %d", head_reduce);
+    OKV_REQUIRE(normalise == OKV_NORM_RAW || normalise == OKV_NORM_SOFTMAX, OKV_ERR_INVALID,
+                "bad normalise %d", normalise);
+  } else {
+    max_score_len = 0;
+    score_lens = nullptr;
+  }
+  AttnWorkspace w;
+  rc = carve_attn_workspace(ws, ws_bytes, batch, layout->num_q_heads, layout->num_kv_heads,
+                            layout->head_dim, max_seq_len, 0, max_score_len, true,
+                            scores != nullptr, &w);
+  if (rc) return rc;
+  RowList r;
+  fill_main(&r, k_base, v_base, layout);
+  r.main_lens = seq_lens;
+  r.max_main_len = max_seq_len;
+  r.score_lens = score_lens;
+  r.max_score_len = max_score_len;
+  return launch_attention(q, r, layout, batch, scale, out, true, head_reduce, normalise, scores,
+                          score_stride, w, (hipStream_t)stream);
+}
+
+int okv_sparse_attn(const void* q, const void* k_base, const void* v_base,
+                    const okv_kv_layout_t* layout, const int32_t* idx, int64_t idx_stride,
+                    const int32_t* sel_lens, int32_t max_sel_len, const void* tail_k,
+                    const void* tail_v, int64_t tail_token_stride, int64_t tail_head_stride,
+                    int64_t tail_batch_stride, const int32_t* tail_lens, int32_t max_tail_len,
+                    int32_t batch, float scale, void* out, void* ws, size_t ws_bytes,
+                    okv_stream_t stream) {
+  int rc = validate_layout(layout, k_base, v_base);
+  if (rc) return rc;
+  OKV_REQUIRE(q && out && v_base, OKV_ERR_INVALID, "q, v_base or out is NULL");
+  OKV_REQUIRE(batch >= 1 && max_sel_len >= 0 && max_tail_len >= 0, OKV_ERR_INVALID,
+              "bad batch or length");
+  OKV_REQUIRE(max_sel_len + max_tail_len >= 1, OKV_ERR_INVALID, "no rows to attend to");
+  if (idx) OKV_REQUIRE(idx_stride >= max_sel_len, OKV_ERR_INVALID, "idx_stride < max_sel_len");
+  if (max_tail_len > 0) {
+    OKV_REQUIRE(tail_k && tail_v, OKV_ERR_INVALID, "tail pointers are NULL");
+    OKV_REQUIRE(((uintptr_t)tail_k & 15) == 0 && ((uintptr_t)tail_v & 15) == 0, OKV_ERR_INVALID,
+                "tail pointers must be 16-byte aligned");
+    OKV_REQUIRE(tail_token_stride % 8 == 0 && tail_head_stride % 8 == 0 &&
+                    tail_batch_stride % 8 == 0,
+                OKV_ERR_INVALID, "tail strides must be multiples of 8 elements");
+  }
+  AttnWorkspace w;
+  rc = carve_attn_workspace(ws, ws_bytes, batch, layout->num_q_heads, layout->num_kv_heads,
+                            layout->head_dim, max_sel_len, max_tail_len, 0, true, false, &w);
+  if (rc) return rc;
+  RowList r;
+  fill_main(&r, k_base, v_base, layout);
+  r.idx = idx;
+  r.idx_stride = idx_stride;
+  r.main_lens = sel_lens;
+  r.max_main_len = max_sel_len;
+  r.tail_k = tail_k;
+  r.tail_v = tail_v;
+  r.tail_token_stride = tail_token_stride;
+  r.tail_head_stride = tail_head_stride;
+  r.tail_batch_stride = tail_batch_stride;
+  r.tail_lens = tail_lens;
+  r.max_tail_len = max_tail_len;
+  return launch_attention(q, r, layout, batch, scale, out, true, 0, 0, nullptr, 0, w,
+                          (hipStream_t)stream);
+}
+
+}  // extern "C"

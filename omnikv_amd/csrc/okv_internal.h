@@ -1,0 +1,134 @@
+// Shared declarations of libomnikv_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/omnikv_hip.h"
+
+namespace okv {
+
+// ---------------------------------------------------------------- errors
+void set_error(const char* fmt, ...);
+
+#define OKV_REQUIRE(cond, code, ...) \
+  do {                               \
+    if (!(cond)) {                   \
+      okv::set_error(__VA_ARGS__);   \
+      return (code);                 \
+    }                                \
+  } while (0)
+
+#define OKV_HIP_CHECK(expr)                                                      \
+  do {                                                                           \
+    hipError_t e_ = (expr);                                                      \
+    if (e_ != hipSuccess) {                                                      \
+      okv::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_),      \
+                     __FILE__, __LINE__);                                        \
+      return OKV_ERR_HIP;                                                        \
+    }                                                                            \
+  } while (0)
+
+// ---------------------------------------------------------------- row lists
+// One request's rows as the attention / scoring kernels see them: a main
+// segment (all cached tokens, or the selected ones through idx) followed by an
+// optional tail segment held in a separate buffer.
+struct RowList {
+  const void* k_base;
+  const void* v_base;
+  int64_t token_stride, head_stride, batch_stride;  // elements
+  const int32_t* page_table;
+  int32_t page_size, page_table_stride;
+  int64_t page_stride;
+  const int32_t* idx;  // optional indirection of the main segment
+  int64_t idx_stride;
+  const int32_t* main_lens;  // optional per-request lengths
+  int32_t max_main_len;
+  const void* tail_k;
+  const void* tail_v;
+  int64_t tail_token_stride, tail_head_stride, tail_batch_stride;
+  const int32_t* tail_lens;
+  int32_t max_tail_len;
+  const int32_t* score_lens;  // rows [0, score_len) are scored; 0 = no scoring
+  int32_t max_score_len;
+};
+
+__device__ __forceinline__ int rl_main_len(const RowList& r, int b) {
+  return r.main_lens ? r.main_lens[b] : r.max_main_len;
+}
+__device__ __forceinline__ int rl_tail_len(const RowList& r, int b) {
+  return r.tail_lens ? r.tail_lens[b] : r.max_tail_len;
+}
+__device__ __forceinline__ int rl_score_len(const RowList& r, int b) {
+  int s = r.score_lens ? r.score_lens[b] : r.max_score_len;
+  int m = rl_main_len(r, b);
+  return s < m ? s : m;
+}
+
+// Splits tile the scored rows [0, A) and the remaining rows [A, L) separately so
+// that no split straddles the scoring boundary.
+__device__ __forceinline__ void rl_split_range(int split, int split_rows, int A, int L,
+                                               int* begin, int* end) {
+  int nA = (A + split_rows - 1) / split_rows;
+  if (split < nA) {
+    *begin = split * split_rows;
+    int e = *begin + split_rows;
+    *end = e < A ? e : A;
+  } else {
+    *begin = A + (split - nA) * split_rows;
+    int e = *begin + split_rows;
+    *end = e < L ? e : L;
+  }
+}
+__host__ __device__ __forceinline__ int rl_num_splits(int split_rows, int A, int L) {
+  return (A + split_rows - 1) / split_rows + (L - A + split_rows - 1) / split_rows;
+}
+
+// Element offset of logical row `row` (kv head 0, d 0) and which buffer it is in.
+__device__ __forceinline__ int64_t rl_row_offset(const RowList& r, int b, int row,
+                                                 int main_len, bool* in_tail) {
+  if (row >= main_len) {
+    *in_tail = true;
+    return (int64_t)b * r.tail_batch_stride + (int64_t)(row - main_len) * r.tail_token_stride;
+  }
+  *in_tail = false;
+  int t = r.idx ? r.idx[(int64_t)b * r.idx_stride + row] : row;
+  if (r.page_table) {
+    int page = r.page_table[(int64_t)b * r.page_table_stride + t / r.page_size];
+    return (int64_t)page * r.page_stride + (int64_t)(t % r.page_size) * r.token_stride;
+  }
+  return (int64_t)b * r.batch_stride + (int64_t)t * r.token_stride;
+}
+
+// 16-byte units in one 128-element row of `esize`-byte elements.
+__host__ __device__ __forceinline__ int kHeadDimBytes16(int esize) { return 128 * esize / 16; }
+
+// ---------------------------------------------------------------- workspace
+// Partial results of the split pass, carved from the caller's workspace.
+struct AttnWorkspace {
+  float* part_o;    // [batch][Hq][splits][D]   normalised partial outputs
+  float* part_lse;  // [batch][Hq][splits]      log2-domain log-sum-exp
+  float* logits;    // [batch][Hq][score_stride] scaled logits (natural units)
+  float* score_lse; // [batch][Hq]              log2-domain lse over scored rows
+  int32_t max_splits;
+  int32_t split_rows;
+  int64_t logits_stride;
+};
+
+size_t attn_workspace_bytes(int batch, int hq, int hkv, int d, int max_main, int max_tail,
+                            int max_score, bool with_v, bool with_logits,
+                            int* split_rows, int* max_splits);
+int carve_attn_workspace(void* ws, size_t ws_bytes, int batch, int hq, int hkv, int d,
+                         int max_main, int max_tail, int max_score, bool with_v,
+                         bool with_logits, AttnWorkspace* out);
+
+int validate_layout(const okv_kv_layout_t* layout, const void* k_base, const void* v_base);
+
+// Implemented in okv_attn.hip.
+int launch_attention(const void* q, const RowList& rows, const okv_kv_layout_t* layout,
+                     int batch, float scale, void* out, bool with_v, int head_reduce,
+                     int normalise, float* scores, int64_t score_stride,
+                     const AttnWorkspace& w, hipStream_t stream);
+
+}  // namespace okv

@@ -1,0 +1,260 @@
+"""Torch-tensor front end of the HIP kernels (one function per C entry point).
+
+Tensors stay torch tensors; this module only extracts pointers, strides and the
+current stream and calls libomnikv_hip.so.  K / V are accepted in the reference's
+shape (bsz, num_kv_heads, tokens, head_dim) with ANY strides whose last dimension
+is contiguous, so both the reference's contiguous cache tensors and views of a
+token-major store are read in place.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+from dataclasses import dataclass
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import KVLayout, Shape, check, lib
+
+_DTYPES = {torch.float32: _lib.OKV_F32, torch.bfloat16: _lib.OKV_BF16, torch.float16: _lib.OKV_F16}
+_REDUCE = {"max": _lib.OKV_REDUCE_MAX, "sum": _lib.OKV_REDUCE_SUM}
+_NORM = {"raw": _lib.OKV_NORM_RAW, "softmax": _lib.OKV_NORM_SOFTMAX}
+
+# selector name -> (normalise, head_reduce); modeling/omnikv.py:40-58 plus the
+# benchmark's softmax-sum variant.
+SELECTOR_MODES = {
+    "last": ("raw", "max"),
+    "softmax_before_last": ("softmax", "max"),
+    "softmax_sum_last": ("softmax", "sum"),
+}
+
+
+@dataclass
+class PagedKV:
+    """A paged K/V pool: pool_k / pool_v (num_pages, page_size, Hkv, D) and
+    page_table (bsz, max_pages) int32.  page_size == 1 is a token-slot table."""
+
+    pool_k: torch.Tensor
+    pool_v: torch.Tensor
+    page_table: torch.Tensor
+    page_size: int
+
+
+_workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def _stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _workspace(device, nbytes: int) -> torch.Tensor:
+    """One growing scratch buffer per (device, stream)."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(), _stream_ptr(device))
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def workspace_bytes(op: int, batch: int, hq: int, hkv: int, d: int, max_seq_len: int,
+                    max_tail_len: int = 0, with_scores: bool = False) -> int:
+    shape = Shape(batch, hq, hkv, d, max_seq_len, max_tail_len, int(with_scores))
+    out = C.c_size_t(0)
+    check(lib().okv_workspace_bytes(op, C.byref(shape), C.byref(out)))
+    return out.value
+
+
+def _require_gpu(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a GPU tensor (the HIP path has no CPU fallback)")
+
+
+def _layout(k, v, hq: int):
+    """(layout struct, k ptr, v ptr, batch, tokens) for tensors or a PagedKV."""
+    if isinstance(k, PagedKV):
+        pk = k
+        pool_k, pool_v = pk.pool_k, pk.pool_v
+        if pool_k.dim() != 4 or pool_k.stride(-1) != 1:
+            raise ValueError("pool_k must be (pages, page_size, Hkv, D) with contiguous D")
+        if pool_v is not None and pool_v.stride() != pool_k.stride():
+            raise ValueError("pool_k and pool_v must share strides")
+        pt = pk.page_table
+        if pt.dtype != torch.int32 or pt.dim() != 2 or pt.stride(1) != 1:
+            raise ValueError("page_table must be (bsz, max_pages) int32, rows contiguous")
+        lay = KVLayout(
+            _DTYPES[pool_k.dtype], hq, pool_k.shape[2], pool_k.shape[3],
+            pool_k.stride(1), pool_k.stride(2), 0,
+            pt.data_ptr(), pk.page_size, pt.stride(0), pool_k.stride(0),
+        )
+        return lay, pool_k.data_ptr(), (pool_v.data_ptr() if pool_v is not None else pool_k.data_ptr()), pt.shape[0], None
+    if k.dim() != 4 or k.stride(-1) != 1:
+        raise ValueError("K must be (bsz, Hkv, tokens, D) with a contiguous last dimension")
+    if v is not None and (v.shape != k.shape or v.stride() != k.stride() or v.dtype != k.dtype):
+        raise ValueError("K and V must share shape, strides and dtype")
+    lay = KVLayout(
+        _DTYPES[k.dtype], hq, k.shape[1], k.shape[3],
+        k.stride(2), k.stride(1), k.stride(0), None, 0, 0, 0,
+    )
+    return lay, k.data_ptr(), (v.data_ptr() if v is not None else k.data_ptr()), k.shape[0], k.shape[2]
+
+
+def _q3(q: torch.Tensor) -> torch.Tensor:
+    if q.dim() == 4:
+        if q.shape[2] != 1:
+            raise ValueError("q must hold one query row per head")
+        q = q[:, :, 0, :]
+    return q.contiguous()
+
+
+def _lens(t: Optional[torch.Tensor], batch: int, name: str) -> int:
+    if t is None:
+        return 0
+    if t.dtype != torch.int32 or not t.is_cuda or t.numel() != batch or not t.is_contiguous():
+        raise ValueError(f"{name} must be a contiguous int32 GPU tensor of {batch} entries")
+    return t.data_ptr()
+
+
+def score(q, k, score_len: Optional[int] = None, selector: str = "last", scale: Optional[float] = None,
+          score_lens: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """(bsz, score_len) fp32 filter-layer scores; okv_score."""
+    q = _q3(q)
+    _require_gpu(q, "q")
+    hq, d = q.shape[1], q.shape[2]
+    lay, kp, _, batch, n = _layout(k, None, hq)
+    if score_len is None:
+        if n is None:
+            raise ValueError("score_len is required with a paged pool")
+        score_len = n
+    norm, red = SELECTOR_MODES[selector]
+    if out is None:
+        out = torch.empty((batch, score_len), dtype=torch.float32, device=q.device)
+    nbytes = workspace_bytes(_lib.OKV_OP_SCORE, batch, hq, lay.num_kv_heads, d, score_len)
+    ws = _workspace(q.device, nbytes)
+    check(lib().okv_score(
+        q.data_ptr(), kp, C.byref(lay), _lens(score_lens, batch, "score_lens"), score_len, batch,
+        _REDUCE[red], _NORM[norm], scale if scale is not None else 1.0 / math.sqrt(d),
+        out.data_ptr(), out.stride(0), ws.data_ptr(), ws.numel(), _stream_ptr(q.device)))
+    return out
+
+
+def topk(scores: torch.Tensor, k: int, seq_lens: Optional[torch.Tensor] = None,
+         k_per_seg: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """(bsz, min(k, N)) int32 ascending indices of the k largest scores; okv_topk."""
+    _require_gpu(scores, "scores")
+    if scores.dtype != torch.float32 or scores.dim() != 2 or scores.stride(1) != 1:
+        raise ValueError("scores must be (bsz, N) float32 with contiguous rows")
+    batch, n = scores.shape
+    kk = min(k, n)
+    if out is None:
+        out = torch.empty((batch, kk), dtype=torch.int32, device=scores.device)
+    if kk == 0:
+        return out
+    check(lib().okv_topk(
+        scores.data_ptr(), scores.stride(0), _lens(seq_lens, batch, "seq_lens"), n,
+        _lens(k_per_seg, batch, "k_per_seg"), k, batch, out.data_ptr(), out.stride(0),
+        None, 0, _stream_ptr(scores.device)))
+    return out
+
+
+def dense_attn(q, k, v=None, seq_len: Optional[int] = None, seq_lens: Optional[torch.Tensor] = None,
+               scale: Optional[float] = None, selector: Optional[str] = None,
+               score_len: Optional[int] = None, score_lens: Optional[torch.Tensor] = None):
+    """Dense GQA decode attention; with `selector` also returns the filter-layer
+    scores of the first score_len tokens from the same pass.  okv_dense_attn."""
+    q = _q3(q)
+    _require_gpu(q, "q")
+    hq, d = q.shape[1], q.shape[2]
+    lay, kp, vp, batch, n = _layout(k, v, hq)
+    if seq_len is None:
+        if n is None:
+            raise ValueError("seq_len is required with a paged pool")
+        seq_len = n
+    out = torch.empty_like(q)
+    scores = None
+    sp, ss, red, norm = None, 0, 0, 0
+    if selector is not None:
+        norm_s, red_s = SELECTOR_MODES[selector]
+        red, norm = _REDUCE[red_s], _NORM[norm_s]
+        if score_len is None:
+            score_len = seq_len
+        scores = torch.empty((batch, score_len), dtype=torch.float32, device=q.device)
+        sp, ss = scores.data_ptr(), scores.stride(0)
+    nbytes = workspace_bytes(_lib.OKV_OP_DENSE_ATTN, batch, hq, lay.num_kv_heads, d, seq_len,
+                             with_scores=selector is not None)
+    ws = _workspace(q.device, nbytes)
+    check(lib().okv_dense_attn(
+        q.data_ptr(), kp, vp, C.byref(lay), _lens(seq_lens, batch, "seq_lens"), seq_len, batch,
+        scale if scale is not None else 1.0 / math.sqrt(d), out.data_ptr(),
+        _lens(score_lens, batch, "score_lens"), score_len or 0, red, norm, sp, ss,
+        ws.data_ptr(), ws.numel(), _stream_ptr(q.device)))
+    return (out, scores) if selector is not None else out
+
+
+def sparse_attn(q, k, v=None, idx: Optional[torch.Tensor] = None, sel_len: Optional[int] = None,
+                sel_lens: Optional[torch.Tensor] = None, tail_k: Optional[torch.Tensor] = None,
+                tail_v: Optional[torch.Tensor] = None, tail_len: Optional[int] = None,
+                tail_lens: Optional[torch.Tensor] = None, scale: Optional[float] = None) -> torch.Tensor:
+    """Attention over rows idx of K/V followed by the tail rows; okv_sparse_attn.
+
+    idx (bsz, k) int32 ascending, or None for rows [0, sel_len).  tail_k / tail_v
+    are (bsz, Hkv, T, D) with any strides (last dimension contiguous)."""
+    q = _q3(q)
+    _require_gpu(q, "q")
+    hq, d = q.shape[1], q.shape[2]
+    lay, kp, vp, batch, n = _layout(k, v, hq)
+    ip, istride = None, 0
+    if idx is not None:
+        if idx.dtype != torch.int32 or idx.dim() != 2 or idx.stride(1) != 1 or not idx.is_cuda:
+            raise ValueError("idx must be a (bsz, k) int32 GPU tensor with contiguous rows")
+        ip, istride = idx.data_ptr(), idx.stride(0)
+        if sel_len is None:
+            sel_len = idx.shape[1]
+    elif sel_len is None:
+        sel_len = n
+    tkp = tvp = None
+    tts = ths = tbs = 0
+    if tail_k is not None:
+        if tail_k.dim() != 4 or tail_k.stride(-1) != 1 or tail_v.stride() != tail_k.stride():
+            raise ValueError("tail_k / tail_v must be (bsz, Hkv, T, D), same strides, contiguous D")
+        if tail_k.dtype != q.dtype:
+            raise ValueError("tail dtype differs from q")
+        if tail_len is None:
+            tail_len = tail_k.shape[2]
+        tkp, tvp = tail_k.data_ptr(), tail_v.data_ptr()
+        tts, ths, tbs = tail_k.stride(2), tail_k.stride(1), tail_k.stride(0)
+    tail_len = tail_len or 0
+    out = torch.empty_like(q)
+    nbytes = workspace_bytes(_lib.OKV_OP_SPARSE_ATTN, batch, hq, lay.num_kv_heads, d, sel_len, tail_len)
+    ws = _workspace(q.device, nbytes)
+    check(lib().okv_sparse_attn(
+        q.data_ptr(), kp, vp, C.byref(lay), ip, istride, _lens(sel_lens, batch, "sel_lens"), sel_len,
+        tkp, tvp, tts, ths, tbs, _lens(tail_lens, batch, "tail_lens"), tail_len, batch,
+        scale if scale is not None else 1.0 / math.sqrt(d), out.data_ptr(),
+        ws.data_ptr(), ws.numel(), _stream_ptr(q.device)))
+    return out
+
+
+def gather_rows(src, idx: torch.Tensor, out: Optional[torch.Tensor] = None,
+                sel_lens: Optional[torch.Tensor] = None, hq: Optional[int] = None) -> torch.Tensor:
+    """out[b, g, j, :] = src[b, g, idx[b, j], :]; okv_gather_rows.
+
+    `out` may be any (bsz, Hkv, k, D) tensor with a contiguous last dimension;
+    by default it is token-major storage viewed in that shape."""
+    if idx.dtype != torch.int32 or idx.dim() != 2 or idx.stride(1) != 1 or not idx.is_cuda:
+        raise ValueError("idx must be a (bsz, k) int32 GPU tensor with contiguous rows")
+    probe = src.pool_k if isinstance(src, PagedKV) else src
+    hkv = probe.shape[2] if isinstance(src, PagedKV) else probe.shape[1]
+    lay, sp, _, batch, _ = _layout(src, None, hq or hkv)
+    ksel = idx.shape[1]
+    d = probe.shape[-1]
+    if out is None:
+        out = torch.empty((batch, ksel, hkv, d), dtype=probe.dtype, device=idx.device).permute(0, 2, 1, 3)
+    if out.stride(-1) != 1 or out.shape != (batch, hkv, ksel, d):
+        raise ValueError("out must be (bsz, Hkv, k, D) with a contiguous last dimension")
+    check(lib().okv_gather_rows(
+        sp, C.byref(lay), idx.data_ptr(), idx.stride(0), _lens(sel_lens, batch, "sel_lens"), ksel,
+        batch, out.data_ptr(), out.stride(2), out.stride(1), out.stride(0), _stream_ptr(idx.device)))
+    return out

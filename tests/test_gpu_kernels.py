@@ -1,0 +1,232 @@
+"""GPU parity: HIP kernels (through the C ABI) against the CPU oracle on the same
+seeded inputs.  Bars: indices bit-exact on identical fp32 scores; attention
+outputs within 1e-4 (fp32) / 2e-2 (bf16, fp16) max-abs; scores within 1e-4
+relative to the row's largest magnitude when both sides see the same input values.
+"""
+import math
+
+import pytest
+import torch
+
+from omnikv_amd import ops, synth
+from oracle import okv_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+ATTN_TOL = {torch.float32: 1e-4, torch.bfloat16: 2e-2, torch.float16: 2e-2}
+
+
+def _rel_err(a: torch.Tensor, b: torch.Tensor) -> float:
+    return float((a - b).abs().max() / b.abs().max().clamp_min(1e-30))
+
+
+# ------------------------------------------------------------------ top-k
+def _check_topk(scores_cpu: torch.Tensor, k: int):
+    got = ops.topk(scores_cpu.to(DEV), k).cpu().to(torch.int64)
+    want = orc.select_topk_stable(scores_cpu, k)
+    assert got.shape == want.shape
+    assert torch.equal(got, want)
+    if not orc.has_boundary_tie(scores_cpu, k) and not torch.isnan(scores_cpu).any():
+        assert torch.equal(got, orc.select_topk(scores_cpu, k))
+
+
+@pytest.mark.parametrize("n,k", [(1, 1), (7, 3), (64, 64), (100, 1), (1000, 67), (4096, 274),
+                                 (5000, 4999), (65537, 4391), (131072, 8781), (131072, 8782),
+                                 (450000, 30150)])
+def test_topk_random(n, k):
+    g = torch.Generator().manual_seed(n * 31 + k)
+    _check_topk(torch.randn((1, n), generator=g), k)
+
+
+@pytest.mark.parametrize("levels", [2, 5, 100])
+def test_topk_heavy_ties(levels):
+    g = torch.Generator().manual_seed(levels)
+    s = torch.randint(0, levels, (2, 20000), generator=g).float() * 0.25 - 3.0
+    for k in (1, 100, 1340, 19999):
+        _check_topk(s, k)
+
+
+def test_topk_special_values():
+    n = 3000
+    s = torch.zeros((1, n))
+    _check_topk(s, 17)  # all equal -> [0, 17)
+    assert torch.equal(ops.topk(s.to(DEV), 17).cpu(), torch.arange(17, dtype=torch.int32)[None])
+    s = torch.randn((1, n), generator=torch.Generator().manual_seed(5))
+    s[0, 10] = float("inf")
+    s[0, 11] = float("-inf")
+    s[0, 12] = 0.0
+    s[0, 13] = -0.0
+    s[0, 2000] = float("inf")
+    for k in (1, 2, 3, 1500, n - 1, n):
+        _check_topk(s, k)
+    z = torch.tensor([[0.0, -0.0, 0.0, -0.0, -1.0, -0.0]])
+    assert ops.topk(z.to(DEV), 3).cpu().tolist() == [[0, 1, 2]]  # -0.0 ties with +0.0
+    s[0, 77] = float("nan")
+    s[0, 2999] = float("nan")
+    got = ops.topk(s.to(DEV), 3).cpu()[0].tolist()
+    assert got == [10, 77, 2999]  # NaN ranks above +inf; lowest index wins among the infs
+
+
+def test_topk_narrow_range_and_softmax_scores():
+    g = torch.Generator().manual_seed(9)
+    s = 2.0 + 1e-4 * torch.rand((1, 50000), generator=g)  # keys within a few thousand ulps
+    _check_topk(s, 3350)
+    p = torch.softmax(4.0 * torch.randn((1, 131072), generator=g), dim=-1) * 32
+    _check_topk(p, 8781)
+    neg = -torch.rand((1, 9000), generator=g) - 0.5 + torch.randn((1, 9000), generator=g)
+    _check_topk(neg, 603)
+
+
+def test_topk_ragged_batch():
+    g = torch.Generator().manual_seed(11)
+    lens = torch.tensor([5000, 17, 32768, 1, 9001], dtype=torch.int32)
+    ks = torch.tensor([335, 20, 2195, 1, 0], dtype=torch.int32)
+    nmax = int(lens.max())
+    s = torch.randn((len(lens), nmax), generator=g)
+    out = torch.full((len(lens), int(ks.max())), -7, dtype=torch.int32, device=DEV)
+    ops.topk(s.to(DEV), int(ks.max()), seq_lens=lens.to(DEV), k_per_seg=ks.to(DEV), out=out)
+    out = out.cpu()
+    for b in range(len(lens)):
+        kb = min(int(ks[b]), int(lens[b]))
+        want = orc.select_topk_stable(s[b:b + 1, : int(lens[b])], kb)[0].to(torch.int32)
+        assert torch.equal(out[b, :kb], want)
+        assert (out[b, kb:] == -7).all()  # untouched beyond k_b
+
+
+# ---------------------------------------------------------------- scoring
+def _inputs(n, dtype, layout):
+    q, k, v = synth.filter_layer_inputs(n)
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    kd, vd = k.to(DEV), v.to(DEV)
+    if layout == "token_major":
+        kd, vd = synth.token_major(kd), synth.token_major(vd)
+    return q, k, v, kd, vd
+
+
+@pytest.mark.parametrize("selector", ["last", "softmax_before_last", "softmax_sum_last"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("layout", ["hf", "token_major"])
+def test_score_matches_oracle(selector, dtype, layout):
+    n = 4096
+    q, k, v, kd, vd = _inputs(n, dtype, layout)
+    got = ops.score(q.to(DEV), kd, selector=selector).cpu()
+    want = orc.score_tokens(q.float(), k.float(), n, selector)  # same values, fp32 math
+    assert got.shape == want.shape
+    assert _rel_err(got, want) < 1e-4
+    if "softmax" in selector and "sum" in selector:
+        assert abs(float(got.sum()) - 32.0) < 1e-2  # each head's softmax sums to one
+    # selected sets agree except for scores that differ in the last bits at the cut
+    kk = orc.num_selected_tokens(0.067, n)
+    a = set(ops.topk(got.to(DEV), kk).cpu()[0].tolist())
+    b = set(orc.select_topk(want, kk)[0].tolist())
+    assert len(a & b) >= kk - 2
+
+
+def test_score_partial_length_and_odd_sizes():
+    for n, consider in [(1000, 1000), (1000, 777), (65, 64), (4099, 4099), (300, 1)]:
+        q, k, _ = synth.filter_layer_inputs(n, seed=77)
+        for selector in ("last", "softmax_sum_last"):
+            got = ops.score(q.to(DEV), k.to(DEV), score_len=consider, selector=selector).cpu()
+            want = orc.score_tokens(q, k, consider, selector)
+            assert got.shape == (1, consider)
+            assert _rel_err(got, want) < 1e-4
+
+
+# -------------------------------------------------------------- attention
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("layout", ["hf", "token_major"])
+@pytest.mark.parametrize("n", [1, 63, 4096, 20011])
+def test_dense_attention(dtype, layout, n):
+    q, k, v, kd, vd = _inputs(n, dtype, layout)
+    got = ops.dense_attn(q.to(DEV), kd, vd).cpu().float()
+    want = orc.gqa_attention(q.float(), k.float(), v.float())[:, :, 0, :]
+    assert (got - want).abs().max() < ATTN_TOL[dtype]
+    if dtype != torch.float32:  # and against the oracle run in the low precision itself
+        low = orc.gqa_attention(q, k, v)[:, :, 0, :].float()
+        assert (got - low).abs().max() < 2 * ATTN_TOL[dtype]
+
+
+@pytest.mark.parametrize("selector", ["last", "softmax_before_last", "softmax_sum_last"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_dense_attention_with_fused_scores(selector, dtype):
+    n, consider = 4096 + 37, 4096
+    q, k, v, kd, vd = _inputs(n, dtype, "token_major")
+    out, scores = ops.dense_attn(q.to(DEV), kd, vd, selector=selector, score_len=consider)
+    want_o = orc.gqa_attention(q.float(), k.float(), v.float())[:, :, 0, :]
+    want_s = orc.score_tokens(q.float(), k.float(), consider, selector)
+    assert (out.cpu().float() - want_o).abs().max() < ATTN_TOL[dtype]
+    assert _rel_err(scores.cpu(), want_s) < 1e-4
+    alone = ops.score(q.to(DEV), kd, score_len=consider, selector=selector)
+    assert _rel_err(scores.cpu(), alone.cpu()) < 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("layout", ["hf", "token_major"])
+@pytest.mark.parametrize("n,ksel,tail", [(4096, 274, 0), (4096, 274, 5), (4096, 1, 1), (20000, 1340, 100),
+                                         (512, 512, 3), (300, 0, 7)])
+def test_sparse_attention(dtype, layout, n, ksel, tail):
+    q, k, v, kd, vd = _inputs(n, dtype, layout)
+    g = torch.Generator().manual_seed(n + ksel + tail)
+    idx = torch.sort(torch.randperm(n, generator=g)[:ksel]).values
+    qn = synth.fresh_q().to(dtype)
+    tk = torch.randn((1, 8, tail, 128), generator=g).to(dtype)
+    tv = torch.randn((1, 8, tail, 128), generator=g).to(dtype)
+    pk = torch.cat([orc.gather_rows(k, idx), tk], dim=-2)
+    pv = torch.cat([orc.gather_rows(v, idx), tv], dim=-2)
+    want = orc.gqa_attention(qn.float(), pk.float(), pv.float())[:, :, 0, :]
+    idx_d = idx.to(torch.int32)[None].to(DEV) if ksel > 0 else torch.zeros((1, 0), dtype=torch.int32, device=DEV)
+    got = ops.sparse_attn(qn.to(DEV), kd, vd, idx=idx_d,
+                          tail_k=tk.to(DEV) if tail else None, tail_v=tv.to(DEV) if tail else None)
+    assert (got.cpu().float() - want).abs().max() < ATTN_TOL[dtype]
+    # an already gathered buffer (idx=None) gives the same answer
+    if ksel > 0:
+        got2 = ops.sparse_attn(qn.to(DEV), pk[:, :, :ksel].to(DEV).contiguous(), pv[:, :, :ksel].to(DEV).contiguous(),
+                               tail_k=tk.to(DEV) if tail else None, tail_v=tv.to(DEV) if tail else None)
+        assert (got2.cpu().float() - want).abs().max() < ATTN_TOL[dtype]
+
+
+def test_sparse_with_all_rows_equals_dense():
+    n = 3000
+    q, k, v, kd, vd = _inputs(n, torch.bfloat16, "token_major")
+    idx = torch.arange(n, dtype=torch.int32, device=DEV)[None]
+    a = ops.sparse_attn(q.to(DEV), kd, vd, idx=idx).float()
+    b = ops.dense_attn(q.to(DEV), kd, vd).float()
+    assert (a - b).abs().max() < 1e-2
+
+
+# ----------------------------------------------------------------- gather
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("layout", ["hf", "token_major"])
+def test_gather_rows_bit_exact(dtype, layout):
+    n, ksel = 5000, 335
+    q, k, v, kd, vd = _inputs(n, dtype, layout)
+    idx = torch.sort(torch.randperm(n, generator=torch.Generator().manual_seed(3))[:ksel]).values
+    got = ops.gather_rows(kd, idx.to(torch.int32)[None].to(DEV))
+    assert got.shape == (1, 8, ksel, 128)
+    assert torch.equal(got.cpu(), orc.gather_rows(k, idx))
+    dst = torch.empty((1, 8, ksel, 128), dtype=dtype, device=DEV)  # the reference's own layout
+    ops.gather_rows(vd, idx.to(torch.int32)[None].to(DEV), out=dst)
+    assert torch.equal(dst.cpu(), orc.gather_rows(v, idx))
+
+
+# ------------------------------------------------ the CPU-runnable config, end to end
+@pytest.mark.parametrize("selector", ["last", "softmax_sum_last"])
+def test_filter_layer_op_config0(selector):
+    n = 4096
+    kk = orc.num_selected_tokens(0.067, n)
+    assert kk == 274
+    q, k, v = synth.filter_layer_inputs(n)
+    _, k2, v2 = synth.filter_layer_inputs(n, seed=synth.SEED_DATA + 100)
+    qn = synth.fresh_q()
+    idx_w, scores_w, out_w = orc.filter_layer_op(q, k, v2, k2, qn, kk, selector)
+    scores = ops.score(q.to(DEV), k.to(DEV), selector=selector)
+    idx = ops.topk(scores, kk)
+    out = ops.sparse_attn(qn.to(DEV), k2.to(DEV), v2.to(DEV), idx=idx)
+    # identical fp32 scores -> identical indices
+    assert torch.equal(ops.topk(scores_w.to(DEV), kk).cpu().to(torch.int64), idx_w)
+    # own scores: identical unless two scores at the cut differ only in the last bits
+    same = set(idx.cpu()[0].tolist()) & set(idx_w[0].tolist())
+    assert len(same) >= kk - 1
+    if len(same) == kk:
+        assert (out.cpu() - out_w[:, :, 0, :]).abs().max() < 1e-4
