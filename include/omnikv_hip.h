@@ -95,6 +95,13 @@ const char* okv_strerror(int status);
 const char* okv_last_error(void);
 int okv_version(void);
 
+/* Process-wide tuning switches, for A/B measurements.  "attn_variant": 0 (default)
+ * runs 16-bit attention / scoring on the matrix-core kernel, 1 forces the portable
+ * VALU kernel for every dtype.  "split_rows": rows per split of the attention /
+ * scoring pass, 0 = automatic.  Set options before sizing workspaces.  No reference
+ * counterpart. */
+int okv_set_option(const char* name, int value);
+
 /* Bytes of scratch `op` needs for `shape`.  No reference counterpart: the
  * reference lets torch allocate (alloc_tensor_func in
  * omnikv-lightllm/.../triton_kernel/flash_decoding.py:45-60). */

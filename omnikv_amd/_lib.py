@@ -22,6 +22,7 @@ EXPORTS = (
     "okv_last_error",
     "okv_version",
     "okv_workspace_bytes",
+    "okv_set_option",
     "okv_score",
     "okv_topk",
     "okv_dense_attn",
@@ -76,6 +77,8 @@ def _declare(l):
     l.okv_version.argtypes = []
     l.okv_workspace_bytes.restype = C.c_int
     l.okv_workspace_bytes.argtypes = [C.c_int, C.POINTER(Shape), C.POINTER(sz)]
+    l.okv_set_option.restype = C.c_int
+    l.okv_set_option.argtypes = [C.c_char_p, C.c_int]
     l.okv_score.restype = C.c_int
     l.okv_score.argtypes = [vp, vp, C.POINTER(KVLayout), vp, i32, i32, i32, i32, f32, vp, i64, vp, sz, vp]
     l.okv_topk.restype = C.c_int

@@ -9,7 +9,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
 OUT = os.path.join(PKG, "libomnikv_hip.so")
-SOURCES = ["okv_api.hip", "okv_attn.hip", "okv_topk.hip", "okv_gather.hip"]
+SOURCES = ["okv_api.hip", "okv_attn.hip", "okv_attn_mfma.hip", "okv_topk.hip", "okv_gather.hip"]
 FLAGS = [
     "--offload-arch=gfx950",
     "-O3",
@@ -25,7 +25,7 @@ FLAGS = [
 def build(force: bool = True, verbose: bool = True) -> str:
     srcs = [os.path.join(HERE, s) for s in SOURCES]
     if not force and os.path.exists(OUT):
-        newest = max(os.path.getmtime(p) for p in srcs + [os.path.join(HERE, "okv_internal.h")])
+        newest = max(os.path.getmtime(p) for p in srcs + [os.path.join(HERE, h) for h in ("okv_internal.h", "okv_device.h")])
         if os.path.getmtime(OUT) >= newest:
             return OUT
     cmd = ["hipcc"] + FLAGS + srcs + ["-o", OUT]

@@ -19,7 +19,10 @@ static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; 
 
 // Rows per split: enough blocks to fill 256 CUs several times over for long
 // contexts, never below one 64-row tile group.
+int g_split_rows_override = 0;
+
 static int choose_split_rows(int batch, int hkv, int total_rows) {
+  if (g_split_rows_override > 0) return g_split_rows_override;
   const int64_t target_blocks = 4096;
   int64_t work = (int64_t)total_rows * hkv * (batch > 0 ? batch : 1);
   int64_t rows = (work + target_blocks - 1) / target_blocks;

@@ -11,66 +11,19 @@
 #include <string.h>
 
 #include "okv_internal.h"
+#include "okv_device.h"
 
 namespace okv {
 
-static constexpr float kLog2e = 1.4426950408889634f;
-static constexpr int kD = 128;
-
-struct BF16 {
-  uint16_t v;
-};
-struct F16 {
-  uint16_t v;
-};
-
-// ---- eight consecutive elements -> fp32
-__device__ __forceinline__ void load8(const float* p, float* o) {
-  float4 a = *reinterpret_cast<const float4*>(p);
-  float4 b = *reinterpret_cast<const float4*>(p + 4);
-  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
-  o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
-}
-__device__ __forceinline__ void load8(const BF16* p, float* o) {
-  uint4 u = *reinterpret_cast<const uint4*>(p);
-  o[0] = __uint_as_float(u.x << 16); o[1] = __uint_as_float(u.x & 0xffff0000u);
-  o[2] = __uint_as_float(u.y << 16); o[3] = __uint_as_float(u.y & 0xffff0000u);
-  o[4] = __uint_as_float(u.z << 16); o[5] = __uint_as_float(u.z & 0xffff0000u);
-  o[6] = __uint_as_float(u.w << 16); o[7] = __uint_as_float(u.w & 0xffff0000u);
-}
-__device__ __forceinline__ void load8(const F16* p, float* o) {
-  uint4 u = *reinterpret_cast<const uint4*>(p);
-  const _Float16* h = reinterpret_cast<const _Float16*>(&u);
-#pragma unroll
-  for (int i = 0; i < 8; ++i) o[i] = (float)h[i];
-}
-
-__device__ __forceinline__ void store1(float* p, float v) { *p = v; }
-__device__ __forceinline__ void store1(BF16* p, float v) {
-  uint32_t u = __float_as_uint(v);
-  uint16_t r;
-  if ((u & 0x7fffffffu) > 0x7f800000u) {
-    r = 0x7fc0;  // NaN
-  } else {
-    u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
-    r = (uint16_t)(u >> 16);
-  }
-  p->v = r;
-}
-__device__ __forceinline__ void store1(F16* p, float v) {
-  _Float16 h = (_Float16)v;
-  p->v = *reinterpret_cast<uint16_t*>(&h);
-}
-
 // ----------------------------------------------------------------- stage 1
-// grid (splits, kv heads, batch), 256 threads.  Each group of 16 lanes walks
+// grid (kv heads, splits, batch), 256 threads.  Each group of 16 lanes walks
 // every 16th row of the split, keeping a private online-softmax state for the G
 // q heads of the kv head; the 16 groups of the block are merged at the end.
 template <typename T, int G, bool WITH_V>
 __global__ __launch_bounds__(256) void attn_stage1_generic(const T* __restrict__ q, RowList rows,
                                                            int hq, float scale, AttnWorkspace w,
                                                            int write_logits) {
-  const int split = blockIdx.x, g = blockIdx.y, b = blockIdx.z;
+  const int g = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
   const int main_len = rl_main_len(rows, b);
   const int L = main_len + rl_tail_len(rows, b);
   const int A = rl_score_len(rows, b);
@@ -196,63 +149,127 @@ __global__ __launch_bounds__(256) void attn_stage1_generic(const T* __restrict__
 }
 
 // ------------------------------------------------------------------- merge
-// grid (q heads, batch), 128 threads (one per output element).
+__device__ __forceinline__ float block_reduce_256(float v, bool is_max, float* red) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) {
+    float x = __shfl_xor(v, o);
+    v = is_max ? fmaxf(v, x) : v + x;
+  }
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float r = red[0];
+#pragma unroll
+  for (int x = 1; x < 4; ++x) r = is_max ? fmaxf(r, red[x]) : r + red[x];
+  return r;
+}
+
+// grid (q heads, batch), 256 threads: 32 float4 columns x 8 split lanes.
 template <typename T>
-__global__ __launch_bounds__(128) void attn_merge(RowList rows, int hq, AttnWorkspace w,
+__global__ __launch_bounds__(256) void attn_merge(RowList rows, int hq, AttnWorkspace w,
                                                   T* __restrict__ out, int with_v,
                                                   int with_score_lse) {
-  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  __shared__ float red[4];
+  __shared__ float4 sred[8][32];
+  const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
   const int main_len = rl_main_len(rows, b);
   const int L = main_len + rl_tail_len(rows, b);
   const int A = rl_score_len(rows, b);
   const int ns = rl_num_splits(w.split_rows, A, L);
   const int nA = (A + w.split_rows - 1) / w.split_rows;
   const int64_t ph = (int64_t)(b * hq + h) * w.max_splits;
-  if (with_v) {
-    float M = -INFINITY;
-    for (int s = 0; s < ns; ++s) M = fmaxf(M, w.part_lse[ph + s]);
-    float den = 0.f, num = 0.f;
-    for (int s = 0; s < ns; ++s) {
-      float f = exp2f(w.part_lse[ph + s] - M);
-      den += f;
-      num += f * w.part_o[(ph + s) * kD + d];
-    }
-    store1(out + (int64_t)(b * hq + h) * kD + d, ns > 0 ? num / den : 0.f);
+  const float* lse = w.part_lse + ph;
+
+  if (with_score_lse) {
+    float mx = -INFINITY;
+    for (int s = tid; s < nA; s += 256) mx = fmaxf(mx, lse[s]);
+    const float MA = block_reduce_256(mx, true, red);
+    float sum = 0.f;
+    for (int s = tid; s < nA; s += 256) sum += exp2f(lse[s] - MA);
+    const float denA = block_reduce_256(sum, false, red);
+    if (tid == 0) w.score_lse[b * hq + h] = MA + log2f(denA);
   }
-  if (with_score_lse && d == 0) {
-    float M = -INFINITY;
-    for (int s = 0; s < nA; ++s) M = fmaxf(M, w.part_lse[ph + s]);
-    float den = 0.f;
-    for (int s = 0; s < nA; ++s) den += exp2f(w.part_lse[ph + s] - M);
-    w.score_lse[b * hq + h] = M + log2f(den);
+  if (!with_v) return;
+
+  float mx = -INFINITY;
+  for (int s = tid; s < ns; s += 256) mx = fmaxf(mx, lse[s]);
+  const float M = block_reduce_256(mx, true, red);
+  float sum = 0.f;
+  for (int s = tid; s < ns; s += 256) sum += exp2f(lse[s] - M);
+  const float den = block_reduce_256(sum, false, red);
+
+  const int dq = tid & 31, sl = tid >> 5;
+  const float4* po = reinterpret_cast<const float4*>(w.part_o + ph * kD) + dq;
+  float4 num = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 4
+  for (int s = sl; s < ns; s += 8) {
+    const float f = exp2f(lse[s] - M);
+    const float4 o = po[(int64_t)s * 32];
+    num.x = fmaf(f, o.x, num.x);
+    num.y = fmaf(f, o.y, num.y);
+    num.z = fmaf(f, o.z, num.z);
+    num.w = fmaf(f, o.w, num.w);
+  }
+  sred[sl][dq] = num;
+  __syncthreads();
+  if (tid < kD) {
+    const float* sr = reinterpret_cast<const float*>(&sred[0][0]);
+    float a = 0.f;
+#pragma unroll
+    for (int x = 0; x < 8; ++x) a += sr[x * kD + tid];
+    store1(out + (int64_t)(b * hq + h) * kD + tid, ns > 0 ? a / den : 0.f);
   }
 }
 
 // ------------------------------------------------------------ score finish
-// grid (ceil(max_score/256), batch), 256 threads, one token each.
+// grid (ceil(max_score/1024), batch), 256 threads, four consecutive tokens each.
 __global__ __launch_bounds__(256) void score_finish(RowList rows, int hq, AttnWorkspace w,
                                                     int head_reduce, int normalise,
                                                     float* __restrict__ scores,
                                                     int64_t score_stride) {
   const int b = blockIdx.y;
-  const int t = blockIdx.x * 256 + threadIdx.x;
+  const int t0 = (blockIdx.x * 256 + threadIdx.x) * 4;
   const int A = rl_score_len(rows, b);
-  if (t >= A) return;
-  float acc = head_reduce == OKV_REDUCE_MAX ? -INFINITY : 0.f;
+  if (t0 >= A) return;
+  const bool is_max = head_reduce == OKV_REDUCE_MAX;
+  const bool soft = normalise == OKV_NORM_SOFTMAX;
+  const float init = is_max ? -INFINITY : 0.f;
+  float acc[4] = {init, init, init, init};
+  const float* lg = w.logits + (int64_t)b * hq * w.logits_stride + t0;
+#pragma unroll 8
   for (int h = 0; h < hq; ++h) {
-    float v = w.logits[(int64_t)(b * hq + h) * w.logits_stride + t];
-    if (normalise == OKV_NORM_SOFTMAX) v = exp2f(v * kLog2e - w.score_lse[b * hq + h]);
-    acc = head_reduce == OKV_REDUCE_MAX ? fmaxf(acc, v) : acc + v;
+    const float4 v4 = *reinterpret_cast<const float4*>(lg + (int64_t)h * w.logits_stride);
+    float v[4] = {v4.x, v4.y, v4.z, v4.w};
+    const float lse = soft ? w.score_lse[b * hq + h] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float x = soft ? exp2f(v[i] * kLog2e - lse) : v[i];
+      acc[i] = is_max ? fmaxf(acc[i], x) : acc[i] + x;
+    }
   }
-  scores[(int64_t)b * score_stride + t] = acc;
+  float* sp = scores + (int64_t)b * score_stride + t0;
+  if (t0 + 3 < A && (((uintptr_t)sp) & 15) == 0) {
+    *reinterpret_cast<float4*>(sp) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (t0 + i < A) sp[i] = acc[i];
+  }
 }
 
 // ----------------------------------------------------------------- launch
+int g_attn_variant = 0;  // 0 = pick per dtype, 1 = portable VALU stage 1 everywhere
+
+bool launch_stage1_mfma(int dtype, const void* q, const RowList& rows, int hq, int hkv, int batch,
+                        float scale, const AttnWorkspace& w, bool with_v, bool write_logits,
+                        hipStream_t stream);
+
 template <typename T, int G>
 static void launch_stage1(const void* q, const RowList& rows, int hq, int hkv, int batch,
                           float scale, const AttnWorkspace& w, bool with_v, bool write_logits,
                           hipStream_t stream) {
-  dim3 grid(w.max_splits, hkv, batch);
+  dim3 grid(hkv, w.max_splits, batch);  // kv head fastest: co-resident blocks cover whole token rows
   if (with_v)
     hipLaunchKernelGGL((attn_stage1_generic<T, G, true>), grid, dim3(256), 0, stream,
                        (const T*)q, rows, hq, scale, w, (int)write_logits);
@@ -268,6 +285,10 @@ static int launch_typed(const void* q, const RowList& rows, const okv_kv_layout_
                         const AttnWorkspace& w, hipStream_t stream) {
   const int hq = lay->num_q_heads, hkv = lay->num_kv_heads, G = hq / hkv;
   const bool want_scores = scores != nullptr;
+  if (g_attn_variant != 1 &&
+      launch_stage1_mfma(lay->dtype, q, rows, hq, hkv, batch, scale, w, with_v, want_scores, stream)) {
+    // 16-bit K/V: stage 1 ran on the matrix-core kernel
+  } else
   switch (G) {
     case 1: launch_stage1<T, 1>(q, rows, hq, hkv, batch, scale, w, with_v, want_scores, stream); break;
     case 2: launch_stage1<T, 2>(q, rows, hq, hkv, batch, scale, w, with_v, want_scores, stream); break;
@@ -277,10 +298,10 @@ static int launch_typed(const void* q, const RowList& rows, const okv_kv_layout_
   }
   const bool need_score_lse = want_scores && normalise == OKV_NORM_SOFTMAX;
   if (with_v || need_score_lse)
-    hipLaunchKernelGGL((attn_merge<T>), dim3(hq, batch), dim3(128), 0, stream, rows, hq, w,
+    hipLaunchKernelGGL((attn_merge<T>), dim3(hq, batch), dim3(256), 0, stream, rows, hq, w,
                        (T*)out, (int)with_v, (int)need_score_lse);
   if (want_scores && rows.max_score_len > 0)
-    hipLaunchKernelGGL(score_finish, dim3((rows.max_score_len + 255) / 256, batch), dim3(256), 0,
+    hipLaunchKernelGGL(score_finish, dim3((rows.max_score_len + 1023) / 1024, batch), dim3(256), 0,
                        stream, rows, hq, w, head_reduce, normalise, scores, score_stride);
   OKV_HIP_CHECK(hipGetLastError());
   return OKV_OK;
@@ -323,6 +344,23 @@ static void fill_main(RowList* r, const void* k, const void* v, const okv_kv_lay
 using namespace okv;
 
 extern "C" {
+
+int okv_set_option(const char* name, int value) {
+  OKV_REQUIRE(name != nullptr, OKV_ERR_INVALID, "option name is NULL");
+  if (strcmp(name, "attn_variant") == 0) {
+    OKV_REQUIRE(value == 0 || value == 1, OKV_ERR_INVALID, "attn_variant must be 0 or 1");
+    g_attn_variant = value;
+    return OKV_OK;
+  }
+  if (strcmp(name, "split_rows") == 0) {
+    OKV_REQUIRE(value == 0 || (value >= 64 && value <= 8192 && value % 64 == 0), OKV_ERR_INVALID,
+                "split_rows must be 0 (automatic) or a multiple of 64 in [64, 8192]");
+    g_split_rows_override = value;
+    return OKV_OK;
+  }
+  set_error("unknown option %s", name);
+  return OKV_ERR_INVALID;
+}
 
 int okv_score(const void* q, const void* k_base, const okv_kv_layout_t* layout,
               const int32_t* score_lens, int32_t max_score_len, int32_t batch,

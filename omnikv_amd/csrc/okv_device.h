@@ -1,0 +1,71 @@
+// Device-side element types and conversions shared by the attention kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace okv {
+
+static constexpr float kLog2e = 1.4426950408889634f;
+static constexpr int kD = 128;
+
+struct BF16 {
+  uint16_t v;
+};
+struct F16 {
+  uint16_t v;
+};
+
+// ---- eight consecutive elements -> fp32
+__device__ __forceinline__ void load8(const float* p, float* o) {
+  float4 a = *reinterpret_cast<const float4*>(p);
+  float4 b = *reinterpret_cast<const float4*>(p + 4);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+  o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+__device__ __forceinline__ void load8(const BF16* p, float* o) {
+  uint4 u = *reinterpret_cast<const uint4*>(p);
+  o[0] = __uint_as_float(u.x << 16); o[1] = __uint_as_float(u.x & 0xffff0000u);
+  o[2] = __uint_as_float(u.y << 16); o[3] = __uint_as_float(u.y & 0xffff0000u);
+  o[4] = __uint_as_float(u.z << 16); o[5] = __uint_as_float(u.z & 0xffff0000u);
+  o[6] = __uint_as_float(u.w << 16); o[7] = __uint_as_float(u.w & 0xffff0000u);
+}
+__device__ __forceinline__ void load8(const F16* p, float* o) {
+  uint4 u = *reinterpret_cast<const uint4*>(p);
+  const _Float16* h = reinterpret_cast<const _Float16*>(&u);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = (float)h[i];
+}
+
+__device__ __forceinline__ void store1(float* p, float v) { *p = v; }
+__device__ __forceinline__ void store1(BF16* p, float v) {
+  uint32_t u = __float_as_uint(v);
+  uint16_t r;
+  if ((u & 0x7fffffffu) > 0x7f800000u) {
+    r = 0x7fc0;  // NaN
+  } else {
+    u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
+    r = (uint16_t)(u >> 16);
+  }
+  p->v = r;
+}
+__device__ __forceinline__ void store1(F16* p, float v) {
+  _Float16 h = (_Float16)v;
+  p->v = *reinterpret_cast<uint16_t*>(&h);
+}
+
+
+// 16 raw bytes (eight 16-bit elements) -> fp32
+__device__ __forceinline__ void cvt8(const BF16*, const uint4& u, float* o) {
+  o[0] = __uint_as_float(u.x << 16); o[1] = __uint_as_float(u.x & 0xffff0000u);
+  o[2] = __uint_as_float(u.y << 16); o[3] = __uint_as_float(u.y & 0xffff0000u);
+  o[4] = __uint_as_float(u.z << 16); o[5] = __uint_as_float(u.z & 0xffff0000u);
+  o[6] = __uint_as_float(u.w << 16); o[7] = __uint_as_float(u.w & 0xffff0000u);
+}
+__device__ __forceinline__ void cvt8(const F16*, const uint4& u, float* o) {
+  const _Float16* h = reinterpret_cast<const _Float16*>(&u);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = (float)h[i];
+}
+
+}  // namespace okv

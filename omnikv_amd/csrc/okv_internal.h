@@ -123,6 +123,8 @@ int carve_attn_workspace(void* ws, size_t ws_bytes, int batch, int hq, int hkv, 
                          int max_main, int max_tail, int max_score, bool with_v,
                          bool with_logits, AttnWorkspace* out);
 
+extern int g_split_rows_override;  // 0 = automatic
+
 int validate_layout(const okv_kv_layout_t* layout, const void* k_base, const void* v_base);
 
 // Implemented in okv_attn.hip.

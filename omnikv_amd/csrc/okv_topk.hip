@@ -81,6 +81,31 @@ __device__ void find_bin(TopkShared& sh, int nbins, uint32_t want, uint32_t* bin
   __syncthreads();
 }
 
+// Calls fn(key) for every score of the request, sixteen loads in flight per thread.
+template <typename F>
+__device__ __forceinline__ void for_each_key(const float* __restrict__ s, int n, F fn) {
+  const int tid = threadIdx.x;
+  int done = 0;
+  if ((((uintptr_t)s) & 15) == 0) {
+    const float4* s4 = reinterpret_cast<const float4*>(s);
+    const int nvec = n >> 2;
+    int i = tid;
+    for (; i + 3 * kThreads < nvec; i += 4 * kThreads) {
+      const float4 a = s4[i], b = s4[i + kThreads], c = s4[i + 2 * kThreads], d = s4[i + 3 * kThreads];
+      fn(score_key(a.x)); fn(score_key(a.y)); fn(score_key(a.z)); fn(score_key(a.w));
+      fn(score_key(b.x)); fn(score_key(b.y)); fn(score_key(b.z)); fn(score_key(b.w));
+      fn(score_key(c.x)); fn(score_key(c.y)); fn(score_key(c.z)); fn(score_key(c.w));
+      fn(score_key(d.x)); fn(score_key(d.y)); fn(score_key(d.z)); fn(score_key(d.w));
+    }
+    for (; i < nvec; i += kThreads) {
+      const float4 a = s4[i];
+      fn(score_key(a.x)); fn(score_key(a.y)); fn(score_key(a.z)); fn(score_key(a.w));
+    }
+    done = nvec << 2;
+  }
+  for (int i = done + tid; i < n; i += kThreads) fn(score_key(s[i]));
+}
+
 __device__ __forceinline__ void clear_hist(TopkShared& sh, int nbins) {
   for (int i = threadIdx.x; i < nbins; i += kThreads) sh.hist[i] = 0;
   __syncthreads();
@@ -109,11 +134,10 @@ __global__ __launch_bounds__(kThreads) void topk_select(const float* __restrict_
 
   // ---- pass 0: key range
   uint32_t kmin = 0xffffffffu, kmax = 0;
-  for (int i = tid; i < n; i += kThreads) {
-    uint32_t key = score_key(s[i]);
+  for_each_key(s, n, [&](uint32_t key) {
     kmin = key < kmin ? key : kmin;
     kmax = key > kmax ? key : kmax;
-  }
+  });
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) {
     uint32_t a = __shfl_xor(kmin, o), c = __shfl_xor(kmax, o);
@@ -144,8 +168,7 @@ __global__ __launch_bounds__(kThreads) void topk_select(const float* __restrict_
     int shift0 = 0;
     while ((range >> shift0) >= (uint32_t)kBins) ++shift0;
     clear_hist(sh, kBins);
-    for (int i = tid; i < n; i += kThreads)
-      atomicAdd(&sh.hist[(score_key(s[i]) - kmin) >> shift0], 1u);
+    for_each_key(s, n, [&](uint32_t key) { atomicAdd(&sh.hist[(key - kmin) >> shift0], 1u); });
     uint32_t bin0, want, cnt;
     find_bin(sh, kBins, (uint32_t)k, &bin0, &want, &cnt);
     // keys of bin0 are kmin + [bin0 << shift0, (bin0+1) << shift0)
@@ -157,13 +180,13 @@ __global__ __launch_bounds__(kThreads) void topk_select(const float* __restrict_
       // ---- pull the candidates (low bits only) into LDS
       if (tid == 0) sh.bcast[4] = 0;
       __syncthreads();
-      for (int i = tid; i < n; i += kThreads) {
-        uint32_t rel = score_key(s[i]) - kmin;
+      for_each_key(s, n, [&](uint32_t key) {
+        const uint32_t rel = key - kmin;
         if ((rel >> shift0) == bin0) {
           uint32_t pos = atomicAdd(&sh.bcast[4], 1u);
           sh.cand[pos] = rel & ((1u << shift0) - 1u);
         }
-      }
+      });
       __syncthreads();
       const int nc = (int)cnt;
       // descend the remaining shift0 bits, up to 11 at a time
@@ -193,11 +216,11 @@ __global__ __launch_bounds__(kThreads) void topk_select(const float* __restrict_
         const int bits = rem > 11 ? 11 : rem;
         const int sh_r = rem - bits;
         clear_hist(sh, 1 << bits);
-        for (int i = tid; i < n; i += kThreads) {
-          uint32_t rel = score_key(s[i]) - kmin;
+        for_each_key(s, n, [&](uint32_t key) {
+          const uint32_t rel = key - kmin;
           if ((rel >> rem) == prefix)
             atomicAdd(&sh.hist[(rel >> sh_r) & ((1u << bits) - 1u)], 1u);
-        }
+        });
         uint32_t bsel, cnt2;
         find_bin(sh, 1 << bits, want, &bsel, &want, &cnt2);
         prefix = (prefix << bits) | bsel;
@@ -209,15 +232,29 @@ __global__ __launch_bounds__(kThreads) void topk_select(const float* __restrict_
   }
 
   // ---- ordered compaction: 4 consecutive tokens per thread per chunk
+  const bool vec = (((uintptr_t)s) & 15) == 0;
+  auto load_chunk = [&](int base, float (&x)[4]) {
+    const int i0 = base + tid * 4;
+    if (vec && i0 + 3 < n) {
+      const float4 a = *reinterpret_cast<const float4*>(s + i0);
+      x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) x[j] = (i0 + j < n) ? s[i0 + j] : 0.f;
+    }
+  };
   uint32_t run_gt = 0, run_eq = 0;  // selected-so-far counts before this chunk
+  float cur[4], nxt[4];
+  load_chunk(0, cur);
   for (int base = 0; base < n; base += kThreads * 4) {
+    if (base + kThreads * 4 < n) load_chunk(base + kThreads * 4, nxt);
     const int i0 = base + tid * 4;
     uint32_t gt[4], eq[4];
     uint32_t cgt = 0, ceq = 0;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      uint32_t key = (i0 + j < n) ? score_key(s[i0 + j]) : 0u;
-      bool valid = i0 + j < n;
+      const bool valid = i0 + j < n;
+      const uint32_t key = score_key(cur[j]);
       gt[j] = valid && key > T;
       eq[j] = valid && key == T;
       cgt += gt[j];
@@ -254,6 +291,8 @@ __global__ __launch_bounds__(kThreads) void topk_select(const float* __restrict_
     }
     run_gt += total & 0xffffu;
     run_eq += total >> 16;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) cur[j] = nxt[j];
   }
 }
 
