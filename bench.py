@@ -182,6 +182,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--detail", action="store_true", help="print per-op timings to stderr")
+    ap.add_argument("--split-rows", type=int, default=0, help="override rows per split (0 = automatic)")
+    ap.add_argument("--attn-variant", type=int, default=0, help="1 = portable VALU stage 1 for every dtype")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -191,7 +193,10 @@ def main():
         sys.exit(2)
 
     from omnikv_amd import ops
+    from omnikv_amd._lib import check, lib
 
+    check(lib().okv_set_option(b"split_rows", args.split_rows))
+    check(lib().okv_set_option(b"attn_variant", args.attn_variant))
     device = torch.device("cuda:0")
     dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[args.dtype]
     esize = 4 if dtype == torch.float32 else 2

@@ -21,22 +21,41 @@ static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; 
 // contexts, never below one 64-row tile group.
 int g_split_rows_override = 0;
 
-static int choose_split_rows(int batch, int hkv, int total_rows) {
+static int num_compute_units() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      cus = n;
+    else
+      cus = 256;  // MI355X
+  }
+  return cus;
+}
+
+// Rows per split.  The pass is bandwidth-bound, so the grid is sized to what the
+// chip holds at once (resident workgroups per CU: 3 with V, 6 for scoring alone),
+// every workgroup getting the same share of rows: all of them start together and
+// finish together, in one round when the split fits the row cap, else in the fewest
+// equal rounds.  The cap keeps the LDS staging of a scored split's logits small.
+static int choose_split_rows(int batch, int hkv, int total_rows, bool with_v, bool with_logits) {
   if (g_split_rows_override > 0) return g_split_rows_override;
-  const int64_t target_blocks = 4096;
-  int64_t work = (int64_t)total_rows * hkv * (batch > 0 ? batch : 1);
-  int64_t rows = (work + target_blocks - 1) / target_blocks;
-  rows = (rows + 63) / 64 * 64;
-  if (rows < 64) rows = 64;
-  if (rows > 1024) rows = 1024;
-  return (int)rows;
+  const int64_t capacity = (int64_t)num_compute_units() * (with_v ? 3 : 6);
+  const int64_t cap_rows = with_logits ? 1024 : 4096;
+  const int64_t work = (int64_t)(total_rows > 0 ? total_rows : 1) * hkv * (batch > 0 ? batch : 1);
+  for (int64_t rounds = 1;; ++rounds) {
+    int64_t rows = (work + rounds * capacity - 1) / (rounds * capacity);
+    rows = (rows + 63) / 64 * 64;
+    if (rows <= cap_rows) return (int)rows;
+  }
 }
 
 size_t attn_workspace_bytes(int batch, int hq, int hkv, int d, int max_main, int max_tail,
                             int max_score, bool with_v, bool with_logits, int* split_rows,
                             int* max_splits) {
   int L = max_main + max_tail;
-  int C = choose_split_rows(batch, hkv, L);
+  int C = choose_split_rows(batch, hkv, L, with_v, with_logits);
   int S = (L + C - 1) / C + (max_score > 0 ? 1 : 0);
   if (S < 1) S = 1;
   if (split_rows) *split_rows = C;

@@ -149,76 +149,77 @@ __global__ __launch_bounds__(256) void attn_stage1_generic(const T* __restrict__
 }
 
 // ------------------------------------------------------------------- merge
-__device__ __forceinline__ float block_reduce_256(float v, bool is_max, float* red) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) {
-    float x = __shfl_xor(v, o);
-    v = is_max ? fmaxf(v, x) : v + x;
-  }
-  __syncthreads();
-  if (lane == 0) red[wave] = v;
-  __syncthreads();
-  float r = red[0];
-#pragma unroll
-  for (int x = 1; x < 4; ++x) r = is_max ? fmaxf(r, red[x]) : r + red[x];
-  return r;
-}
-
-// grid (q heads, batch), 256 threads: 32 float4 columns x 8 split lanes.
+// grid (q heads, batch), 256 threads: 32 float4 columns x 8 split lanes.  Every
+// thread folds its splits with a running max (all loads independent, one trip to
+// memory), then the 8 split lanes of a column meet in LDS.
 template <typename T>
 __global__ __launch_bounds__(256) void attn_merge(RowList rows, int hq, AttnWorkspace w,
                                                   T* __restrict__ out, int with_v,
                                                   int with_score_lse) {
-  __shared__ float red[4];
-  __shared__ float4 sred[8][32];
+  __shared__ float4 snum[8][32];
+  __shared__ float sm[8], sden[8], smA[8], sdenA[8];
   const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
   const int main_len = rl_main_len(rows, b);
   const int L = main_len + rl_tail_len(rows, b);
   const int A = rl_score_len(rows, b);
   const int ns = rl_num_splits(w.split_rows, A, L);
-  const int nA = (A + w.split_rows - 1) / w.split_rows;
+  const int nA = with_score_lse ? (A + w.split_rows - 1) / w.split_rows : 0;
   const int64_t ph = (int64_t)(b * hq + h) * w.max_splits;
   const float* lse = w.part_lse + ph;
-
-  if (with_score_lse) {
-    float mx = -INFINITY;
-    for (int s = tid; s < nA; s += 256) mx = fmaxf(mx, lse[s]);
-    const float MA = block_reduce_256(mx, true, red);
-    float sum = 0.f;
-    for (int s = tid; s < nA; s += 256) sum += exp2f(lse[s] - MA);
-    const float denA = block_reduce_256(sum, false, red);
-    if (tid == 0) w.score_lse[b * hq + h] = MA + log2f(denA);
-  }
-  if (!with_v) return;
-
-  float mx = -INFINITY;
-  for (int s = tid; s < ns; s += 256) mx = fmaxf(mx, lse[s]);
-  const float M = block_reduce_256(mx, true, red);
-  float sum = 0.f;
-  for (int s = tid; s < ns; s += 256) sum += exp2f(lse[s] - M);
-  const float den = block_reduce_256(sum, false, red);
-
   const int dq = tid & 31, sl = tid >> 5;
   const float4* po = reinterpret_cast<const float4*>(w.part_o + ph * kD) + dq;
+
+  float m = -INFINITY, den = 0.f, mA = -INFINITY, denA = 0.f;
   float4 num = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll 4
   for (int s = sl; s < ns; s += 8) {
-    const float f = exp2f(lse[s] - M);
-    const float4 o = po[(int64_t)s * 32];
-    num.x = fmaf(f, o.x, num.x);
-    num.y = fmaf(f, o.y, num.y);
-    num.z = fmaf(f, o.z, num.z);
-    num.w = fmaf(f, o.w, num.w);
+    const float x = lse[s];
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (with_v) o = po[(int64_t)s * 32];
+    const float mn = fmaxf(m, x);
+    const float a = exp2f(m - mn), f = exp2f(x - mn);
+    den = fmaf(den, a, f);
+    num.x = fmaf(num.x, a, f * o.x);
+    num.y = fmaf(num.y, a, f * o.y);
+    num.z = fmaf(num.z, a, f * o.z);
+    num.w = fmaf(num.w, a, f * o.w);
+    m = mn;
+    if (s < nA) {
+      const float mnA = fmaxf(mA, x);
+      denA = fmaf(denA, exp2f(mA - mnA), exp2f(x - mnA));
+      mA = mnA;
+    }
   }
-  sred[sl][dq] = num;
+  snum[sl][dq] = num;
+  if (dq == 0) {
+    sm[sl] = m;
+    sden[sl] = den;
+    smA[sl] = mA;
+    sdenA[sl] = denA;
+  }
   __syncthreads();
-  if (tid < kD) {
-    const float* sr = reinterpret_cast<const float*>(&sred[0][0]);
-    float a = 0.f;
+  if (with_v && tid < kD) {
+    float M = -INFINITY;
 #pragma unroll
-    for (int x = 0; x < 8; ++x) a += sr[x * kD + tid];
-    store1(out + (int64_t)(b * hq + h) * kD + tid, ns > 0 ? a / den : 0.f);
+    for (int x = 0; x < 8; ++x) M = fmaxf(M, sm[x]);
+    const float* sn = reinterpret_cast<const float*>(&snum[0][0]);
+    float a = 0.f, d = 0.f;
+#pragma unroll
+    for (int x = 0; x < 8; ++x) {
+      const float f = (sm[x] == -INFINITY) ? 0.f : exp2f(sm[x] - M);
+      a = fmaf(sn[x * kD + tid], f, a);
+      d = fmaf(sden[x], f, d);
+    }
+    store1(out + (int64_t)(b * hq + h) * kD + tid, ns > 0 ? a / d : 0.f);
+  }
+  if (with_score_lse && tid == 0) {
+    float M = -INFINITY;
+#pragma unroll
+    for (int x = 0; x < 8; ++x) M = fmaxf(M, smA[x]);
+    float d = 0.f;
+#pragma unroll
+    for (int x = 0; x < 8; ++x) d += (smA[x] == -INFINITY) ? 0.f : sdenA[x] * exp2f(smA[x] - M);
+    w.score_lse[b * hq + h] = M + log2f(d);
   }
 }
 

@@ -7,11 +7,13 @@
 // head are the first G columns of the B operand, the rest zero).  The result leaves
 // lane l holding column (head) l%16 of tile rows 4(l/16) .. +4: the lanes of one
 // 16-lane row hold all heads of the same four rows, so each row of lanes keeps its
-// own online softmax and the probabilities reach the P.V lanes by DPP row
-// broadcasts.  P.V is VALU work: lane l owns output elements 8(l%16) .. +8 and
-// accumulates the four rows of its lane row, reading V fully coalesced (256 bytes
-// per row per 16 lanes).  Next tile's K and V are in flight while the current one
-// is consumed.
+// own online softmax, and the probabilities reach the P.V lanes by DPP row
+// broadcasts.  P.V is VALU work on packed pairs: lane l owns output elements
+// 8(l%16) .. +8 and accumulates the four rows of its lane row with v_dot2 (two rows
+// per instruction, probabilities rounded to the K/V element type as matrix-core
+// attention does), reading V fully coalesced (256 bytes per row per 16 lanes).
+// The rows of tile t+2 are looked up and the K/V of tile t+1 are in flight while
+// tile t is consumed.  The sixteen lane rows of the block meet in LDS at the end.
 #include <math.h>
 
 #include "okv_device.h"
@@ -21,6 +23,9 @@ namespace okv {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 __device__ __forceinline__ f32x4_t mfma16(const BF16*, const uint4& a, const uint4& b, f32x4_t c) {
@@ -31,46 +36,71 @@ __device__ __forceinline__ f32x4_t mfma16(const F16*, const uint4& a, const uint
   return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
                                                 __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
 }
+// two fp32 -> one dword of two 16-bit elements (first argument in the low half)
+__device__ __forceinline__ uint32_t pack2(const BF16*, float a, float b) {
+  f32x2_t x = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2_t));
+}
+__device__ __forceinline__ uint32_t pack2(const F16*, float a, float b) {
+  f32x2_t x = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2_t));
+}
+// acc + v.lo*p.lo + v.hi*p.hi
+__device__ __forceinline__ float dot2(const BF16*, uint32_t v, uint32_t p, float acc) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, v),
+                                         __builtin_bit_cast(bf16x2_t, p), acc, false);
+}
+__device__ __forceinline__ float dot2(const F16*, uint32_t v, uint32_t p, float acc) {
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, v), __builtin_bit_cast(f16x2_t, p), acc,
+                                false);
+}
 
 // value of lane H of the caller's 16-lane row
 template <int H>
-__device__ __forceinline__ float row_bcast(float x) {
-  return __int_as_float(
-      __builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x150 + H, 0xf, 0xf, false));
+__device__ __forceinline__ uint32_t row_bcast(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, 0x150 + H, 0xf, 0xf, true);
 }
 
-template <int H, int G, bool RESCALE>
+template <typename T, int H, int G>
 struct HeadStep {
-  // acc[h][:] (*= alpha_h) += p_h * v[:] for heads H .. G-1
-  static __device__ __forceinline__ void fma(float (&acc)[G][8], float p, const float* v) {
-    const float ph = row_bcast<H>(p);
+  // acc[h][:] += P_h(row pair) . V(row pair) for heads H .. G-1
+  static __device__ __forceinline__ void pv(float (&acc)[G][8], uint32_t p, const uint32_t (&vp)[8]) {
+    const uint32_t ph = row_bcast<H>(p);
 #pragma unroll
-    for (int d = 0; d < 8; ++d) acc[H][d] = fmaf(ph, v[d], acc[H][d]);
-    HeadStep<H + 1, G, RESCALE>::fma(acc, p, v);
+    for (int d = 0; d < 8; ++d) acc[H][d] = dot2((const T*)nullptr, vp[d], ph, acc[H][d]);
+    HeadStep<T, H + 1, G>::pv(acc, p, vp);
   }
   static __device__ __forceinline__ void scale(float (&acc)[G][8], float a) {
-    const float ah = row_bcast<H>(a);
+    const float ah = __uint_as_float(row_bcast<H>(__float_as_uint(a)));
 #pragma unroll
     for (int d = 0; d < 8; ++d) acc[H][d] *= ah;
-    HeadStep<H + 1, G, RESCALE>::scale(acc, a);
+    HeadStep<T, H + 1, G>::scale(acc, a);
   }
 };
-template <int G, bool R>
-struct HeadStep<G, G, R> {
-  static __device__ __forceinline__ void fma(float (&)[G][8], float, const float*) {}
+template <typename T, int G>
+struct HeadStep<T, G, G> {
+  static __device__ __forceinline__ void pv(float (&)[G][8], uint32_t, const uint32_t (&)[8]) {}
   static __device__ __forceinline__ void scale(float (&)[G][8], float) {}
 };
 
+// What a lane needs to know about the rows of a tile before it can address them:
+// the K row (index 0) and its four V rows (1..4).
 struct TileRows {
-  int64_t k_off;     // element offset of this lane's K row (kv head and d included)
-  int64_t v_off[4];  // element offsets of this lane's four V rows
-  bool k_tail, v_tail[4];
+  int32_t tok[5];  // token (or page) the row maps to; raw load results
+  int32_t row[5];  // logical row, clamped into the split
 };
 
-template <typename T, int G, bool WITH_V, bool SIMPLE>
+template <int G>
+__host__ __device__ constexpr int stage1_lds_floats(bool with_v) {
+  return 3 * 16 * G + 16 + (with_v ? 16 * G * kD : 0);
+}
+
+// MODE 0: contiguous rows, no index, no tail.  MODE 1: rows through idx (no page table),
+// optional tail.  MODE 2: anything (page tables, idx or not, tail or not).
+template <typename T, int G, bool WITH_V, int MODE, bool LOGITS>
 __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q, RowList rows,
-                                                        int hq, float scale, AttnWorkspace w,
-                                                        int write_logits) {
+                                                        int hq, float scale, AttnWorkspace w) {
+  extern __shared__ float lds[];
   const int g = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
   const int main_len = rl_main_len(rows, b);
   const int L = main_len + rl_tail_len(rows, b);
@@ -82,207 +112,272 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, j4 = lane >> 4;
 
-  // B operand: q heads of this kv head in columns 0..G-1
+  // B operand: q heads of this kv head in columns 0..G-1, zero beyond
   uint4 qf[4];
+  {
+    const int hcol = r16 < G ? r16 : G - 1;
+    const T* qp = q + ((int64_t)(b * hq + g * G + hcol) * kD + 8 * j4);
 #pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    qf[s] = make_uint4(0, 0, 0, 0);
-    if (r16 < G)
-      qf[s] = *reinterpret_cast<const uint4*>(q + ((int64_t)(b * hq + g * G + r16) * kD + 32 * s + 8 * j4));
+    for (int s = 0; s < 4; ++s) {
+      const uint4 v = *reinterpret_cast<const uint4*>(qp + 32 * s);
+      qf[s] = r16 < G ? v : make_uint4(0, 0, 0, 0);
+    }
   }
 
-  const T* kb = reinterpret_cast<const T*>(rows.k_base);
-  const T* vb = reinterpret_cast<const T*>(rows.v_base);
-  const T* tkb = reinterpret_cast<const T*>(rows.tail_k);
-  const T* tvb = reinterpret_cast<const T*>(rows.tail_v);
-  const int64_t head_off = (int64_t)g * rows.head_stride;
-  const int64_t tail_head_off = (int64_t)g * rows.tail_head_stride;
+  const T* kb = reinterpret_cast<const T*>(rows.k_base) + (int64_t)b * rows.batch_stride +
+                (int64_t)g * rows.head_stride;
+  const T* vb = reinterpret_cast<const T*>(rows.v_base) + (int64_t)b * rows.batch_stride +
+                (int64_t)g * rows.head_stride;
+  const T* tkb = reinterpret_cast<const T*>(rows.tail_k) + (int64_t)b * rows.tail_batch_stride +
+                 (int64_t)g * rows.tail_head_stride;
+  const T* tvb = reinterpret_cast<const T*>(rows.tail_v) + (int64_t)b * rows.tail_batch_stride +
+                 (int64_t)g * rows.tail_head_stride;
+  const T* pkb = reinterpret_cast<const T*>(rows.k_base) + (int64_t)g * rows.head_stride;  // paged
+  const T* pvb = reinterpret_cast<const T*>(rows.v_base) + (int64_t)g * rows.head_stride;
+  const uint32_t ts = (uint32_t)rows.token_stride, tts = (uint32_t)rows.tail_token_stride;
+  const int last = end - 1;
 
+  // ---- which rows a tile touches (issues the index / page-table loads)
+  const int32_t* idx_row = rows.idx + (int64_t)b * rows.idx_stride;
   auto tile_rows = [&](int tbase, TileRows& tr) {
-    const int last = end - 1;
-    int kr = tbase + r16;
-    kr = kr < last ? kr : last;
-    if (SIMPLE) {
-      tr.k_tail = false;
-      tr.k_off = (int64_t)b * rows.batch_stride + (int64_t)kr * rows.token_stride + head_off + 8 * j4;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int vr = tbase + 4 * j4 + i;
-        vr = vr < last ? vr : last;
-        tr.v_tail[i] = false;
-        tr.v_off[i] = (int64_t)b * rows.batch_stride + (int64_t)vr * rows.token_stride + head_off + 8 * r16;
-      }
-    } else {
-      tr.k_off = rl_row_offset(rows, b, kr, main_len, &tr.k_tail) +
-                 (tr.k_tail ? tail_head_off : head_off) + 8 * j4;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int vr = tbase + 4 * j4 + i;
-        vr = vr < last ? vr : last;
-        tr.v_off[i] = rl_row_offset(rows, b, vr, main_len, &tr.v_tail[i]) +
-                      (tr.v_tail[i] ? tail_head_off : head_off) + 8 * r16;
+    for (int x = 0; x < 5; ++x) {
+      int r = x == 0 ? tbase + r16 : tbase + 4 * j4 + (x - 1);
+      r = r < last ? r : last;
+      tr.row[x] = r;
+      if (MODE == 0) {
+        tr.tok[x] = r;
+      } else if (MODE == 1) {  // branch-free: main_len >= 1 is guaranteed by the launcher
+        const int ri = r < main_len ? r : main_len - 1;
+        const int t = idx_row[ri];
+        tr.tok[x] = r < main_len ? t : r - main_len;
+      } else if (r >= main_len) {
+        tr.tok[x] = r - main_len;
+      } else {
+        int t = rows.idx ? idx_row[r] : r;
+        if (rows.page_table) {
+          tr.row[x] = -1 - (t % rows.page_size);  // slot in page, tagged as paged
+          t = rows.page_table[(int64_t)b * rows.page_table_stride + t / rows.page_size];
+        }
+        tr.tok[x] = t;
       }
     }
   };
+  auto row_ptr = [&](const TileRows& tr, int x, bool is_v) -> const T* {
+    if (MODE == 0) return (is_v ? vb : kb) + (uint64_t)(uint32_t)tr.tok[x] * ts;
+    if (MODE == 1) {
+      const bool in_tail = tr.row[x] >= main_len;
+      const T* base = in_tail ? (is_v ? tvb : tkb) : (is_v ? vb : kb);
+      return base + (uint64_t)(uint32_t)tr.tok[x] * (in_tail ? tts : ts);
+    }
+    if (tr.row[x] >= main_len) return (is_v ? tvb : tkb) + (uint64_t)(uint32_t)tr.tok[x] * tts;
+    if (tr.row[x] < 0)
+      return (is_v ? pvb : pkb) + (int64_t)tr.tok[x] * rows.page_stride +
+             (uint64_t)(uint32_t)(-1 - tr.row[x]) * ts;
+    return (is_v ? vb : kb) + (uint64_t)(uint32_t)tr.tok[x] * ts;
+  };
   auto load_tile = [&](const TileRows& tr, uint4 (&kf)[4], uint4 (&vf)[4]) {
-    const T* kp = (tr.k_tail ? tkb : kb) + tr.k_off;
+    const T* kp = row_ptr(tr, 0, false) + 8 * j4;
 #pragma unroll
     for (int s = 0; s < 4; ++s) kf[s] = *reinterpret_cast<const uint4*>(kp + 32 * s);
     if (WITH_V) {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        vf[i] = *reinterpret_cast<const uint4*>((tr.v_tail[i] ? tvb : vb) + tr.v_off[i]);
+        vf[i] = *reinterpret_cast<const uint4*>(row_ptr(tr, 1 + i, true) + 8 * r16);
     }
   };
 
-  float m = -INFINITY, l = 0.f;  // softmax state of (head r16, lane row j4)
-  float acc[G][8];               // output elements 8*r16.. of the rows of lane row j4
+  float m = -INFINITY, l = 0.f;  // softmax state of (head r16, lane row j4); m in raw q.k units
+  float acc[G][8];               // output elements 8*r16.. summed over the rows of lane row j4
 #pragma unroll
   for (int h = 0; h < G; ++h)
 #pragma unroll
     for (int d = 0; d < 8; ++d) acc[h][d] = 0.f;
   const float sl2 = scale * kLog2e;
+  const bool scored = LOGITS && begin < A;  // a scored split ends at or before A
+  float* slog = lds + stage1_lds_floats<G>(WITH_V);  // [G][split_rows] scaled logits of the split
 
   auto compute = [&](int tbase, const uint4 (&kf)[4], const uint4 (&vf)[4]) {
     f32x4_t S = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < 4; ++s) S = mfma16((const T*)nullptr, kf[s], qf[s], S);
     const int row0 = tbase + 4 * j4;
-    if (write_logits && begin < A && r16 < G && row0 < end) {  // a scored split ends at or before A
-      float* lp = w.logits + (int64_t)(b * hq + g * G + r16) * w.logits_stride + row0;
-      if (row0 + 3 < end) {
-        *reinterpret_cast<float4*>(lp) = make_float4(S[0] * scale, S[1] * scale, S[2] * scale, S[3] * scale);
-      } else {
+    const bool partial = tbase + 16 > end;  // wave-uniform
+    if (scored && r16 < G)  // staged in LDS, flushed after the loop: no global store in the loop
+      *reinterpret_cast<float4*>(slog + r16 * w.split_rows + (row0 - begin)) =
+          make_float4(S[0] * scale, S[1] * scale, S[2] * scale, S[3] * scale);
+    float s[4] = {S[0], S[1], S[2], S[3]};
+    if (partial) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (row0 + i < end) lp[i] = S[i] * scale;
-      }
+      for (int i = 0; i < 4; ++i)
+        if (row0 + i >= end) s[i] = -INFINITY;
     }
-    float s2[4];
-    float mt = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      s2[i] = (row0 + i < end) ? S[i] * sl2 : -INFINITY;
-      mt = fmaxf(mt, s2[i]);
-    }
-    const float mn = fmaxf(m, mt);
-    const float ms = (mn == -INFINITY) ? 0.f : mn;
-    const float alpha = exp2f(m - ms);
+    const float mn = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), m);
+    const float ms = (partial && mn == -INFINITY) ? 0.f : mn;
+    const float neg = -ms * sl2;
+    const float alpha = __builtin_amdgcn_exp2f((m - ms) * sl2);  // exactly 1 while the max stands
     float p[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) p[i] = exp2f(s2[i] - ms);
-    l = l * alpha + ((p[0] + p[1]) + (p[2] + p[3]));
+    for (int i = 0; i < 4; ++i) p[i] = __builtin_amdgcn_exp2f(fmaf(s[i], sl2, neg));
+    l = fmaf(l, alpha, (p[0] + p[1]) + (p[2] + p[3]));
+    const bool changed = (r16 < G) && (mn > m);
     m = mn;
     if (WITH_V) {
-      const bool changed = (r16 < G) && (alpha != 1.0f);
-      if (__ballot(changed) != 0ull) HeadStep<0, G, true>::scale(acc, alpha);
+      if (__ballot(changed) != 0ull) HeadStep<T, 0, G>::scale(acc, alpha);
+      const uint32_t p01 = pack2((const T*)nullptr, p[0], p[1]);
+      const uint32_t p23 = pack2((const T*)nullptr, p[2], p[3]);
+      uint32_t vp[8];
+      {
+        const uint32_t a[4] = {vf[0].x, vf[0].y, vf[0].z, vf[0].w};
+        const uint32_t c[4] = {vf[1].x, vf[1].y, vf[1].z, vf[1].w};
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float v[8];
-        cvt8((const T*)nullptr, vf[i], v);
-        HeadStep<0, G, false>::fma(acc, p[i], v);
+        for (int j = 0; j < 4; ++j) {
+          vp[2 * j] = __builtin_amdgcn_perm(c[j], a[j], 0x05040100u);
+          vp[2 * j + 1] = __builtin_amdgcn_perm(c[j], a[j], 0x07060302u);
+        }
+        HeadStep<T, 0, G>::pv(acc, p01, vp);
+      }
+      {
+        const uint32_t a[4] = {vf[2].x, vf[2].y, vf[2].z, vf[2].w};
+        const uint32_t c[4] = {vf[3].x, vf[3].y, vf[3].z, vf[3].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          vp[2 * j] = __builtin_amdgcn_perm(c[j], a[j], 0x05040100u);
+          vp[2 * j + 1] = __builtin_amdgcn_perm(c[j], a[j], 0x07060302u);
+        }
+        HeadStep<T, 0, G>::pv(acc, p23, vp);
       }
     }
   };
 
-  // ---- tiles of this wave: begin + 16*(wave + 4*n), software-pipelined by one tile
-  uint4 kA[4], vA[4], kB[4], vB[4];
-  TileRows tr;
-  int t = begin + wave * 16;
-  if (t < end) {
-    tile_rows(t, tr);
-    load_tile(tr, kA, vA);
-    while (true) {
-      int tn = t + 64;
-      bool more = tn < end;
-      if (more) {
-        tile_rows(tn, tr);
+  // ---- tiles of this wave: begin + 16*(wave + 4*n).  Inside the loop every load is
+  // unconditional (a tile index past the wave's last tile is clamped to it), so the
+  // number of loads in flight is the same on every path and the wait before a tile's
+  // first use leaves the next tile's loads outstanding.
+  {
+    uint4 kA[4], vA[4], kB[4], vB[4];
+    TileRows tr, tr0;
+    int t = begin + wave * 16;
+    if (t < end) {
+      const int t_last = t + ((last - t) >> 6 << 6);
+      tile_rows(t, tr0);
+      if (t == t_last) {  // one tile
+        load_tile(tr0, kA, vA);
+        compute(t, kA, vA);
+      } else if (t + 64 == t_last) {  // two tiles: everything in flight at once, nothing extra
+        tile_rows(t + 64, tr);
+        load_tile(tr0, kA, vA);
         load_tile(tr, kB, vB);
+        compute(t, kA, vA);
+        compute(t + 64, kB, vB);
+      } else {
+        tile_rows(t + 64, tr);  // both lookups leave before the first one is awaited
+        load_tile(tr0, kA, vA);
+        while (true) {
+          load_tile(tr, kB, vB);
+          tile_rows(min(t + 128, t_last), tr);
+          compute(t, kA, vA);
+          t += 64;
+          load_tile(tr, kA, vA);
+          tile_rows(min(t + 128, t_last), tr);
+          compute(t, kB, vB);
+          if (t == t_last) break;
+          t += 64;
+          if (t == t_last) {
+            compute(t, kA, vA);
+            break;
+          }
+        }
       }
-      compute(t, kA, vA);
-      if (!more) break;
-      t = tn;
-      tn = t + 64;
-      more = tn < end;
-      if (more) {
-        tile_rows(tn, tr);
-        load_tile(tr, kA, vA);
-      }
-      compute(t, kB, vB);
-      if (!more) break;
-      t = tn;
     }
   }
 
-  // ---- merge the four lane rows of the wave
-  float M = fmaxf(m, __shfl_xor(m, 16));
-  M = fmaxf(M, __shfl_xor(M, 32));
-  const float f = (m == -INFINITY) ? 0.f : exp2f(m - M);
-  float lw = l * f;
-  lw += __shfl_xor(lw, 16);
-  lw += __shfl_xor(lw, 32);
+  // ---- the 16 lane rows of the block meet in LDS
+  float* sm = lds;                // [16][G] running max (raw units)
+  float* sl = lds + 16 * G;       // [16][G] sum of exp
+  float* sacc = lds + 48 * G + 16;  // [16][G][128]
+  const int grp = wave * 4 + j4;
+  if (r16 < G) {
+    sm[grp * G + r16] = m;
+    sl[grp * G + r16] = l;
+  }
   if (WITH_V) {
-    HeadStep<0, G, true>::scale(acc, f);
 #pragma unroll
-    for (int h = 0; h < G; ++h)
-#pragma unroll
-      for (int d = 0; d < 8; ++d) {
-        float a = acc[h][d];
-        a += __shfl_xor(a, 16);
-        a += __shfl_xor(a, 32);
-        acc[h][d] = a;
-      }
-  }
-
-  // ---- merge the four waves through LDS and write the split's partial
-  __shared__ float sm[4][G];
-  __shared__ float sl[4][G];
-  __shared__ float sacc[WITH_V ? 4 : 1][G][kD];
-  if (j4 == 0) {
-    if (r16 < G) {
-      sm[wave][r16] = M;
-      sl[wave][r16] = lw;
-    }
-    if (WITH_V) {
-#pragma unroll
-      for (int h = 0; h < G; ++h)
-#pragma unroll
-        for (int d = 0; d < 8; ++d) sacc[wave][h][r16 * 8 + d] = acc[h][d];
+    for (int h = 0; h < G; ++h) {
+      float4* dst = reinterpret_cast<float4*>(sacc + (grp * G + h) * kD + r16 * 8);
+      dst[0] = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+      dst[1] = make_float4(acc[h][4], acc[h][5], acc[h][6], acc[h][7]);
     }
   }
   __syncthreads();
+  if (scored) {
+    const int quads = w.split_rows >> 2;
+    for (int o = threadIdx.x; o < G * quads; o += 256) {
+      const int h = o / quads, r = begin + 4 * (o % quads);
+      if (r >= end) continue;
+      const float4 v = *reinterpret_cast<const float4*>(slog + h * w.split_rows + (r - begin));
+      float* lp = w.logits + (int64_t)(b * hq + g * G + h) * w.logits_stride + r;
+      if (r + 3 < end) {
+        *reinterpret_cast<float4*>(lp) = v;
+      } else {
+        lp[0] = v.x;
+        if (r + 1 < end) lp[1] = v.y;
+        if (r + 2 < end) lp[2] = v.z;
+      }
+    }
+  }
   for (int o = threadIdx.x; o < G * kD; o += 256) {
     const int h = o / kD, d = o % kD;
-    const float Mb = fmaxf(fmaxf(sm[0][h], sm[1][h]), fmaxf(sm[2][h], sm[3][h]));
+    float M = -INFINITY;
+#pragma unroll
+    for (int x = 0; x < 16; ++x) M = fmaxf(M, sm[x * G + h]);
     float den = 0.f, num = 0.f;
 #pragma unroll
-    for (int x = 0; x < 4; ++x) {
-      const float fx = (sm[x][h] == -INFINITY) ? 0.f : exp2f(sm[x][h] - Mb);
-      den += sl[x][h] * fx;
-      if (WITH_V) num += sacc[x][h][d] * fx;
+    for (int x = 0; x < 16; ++x) {
+      const float mm = sm[x * G + h];
+      const float fx = (mm == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((mm - M) * sl2);
+      den = fmaf(sl[x * G + h], fx, den);
+      if (WITH_V) num = fmaf(sacc[(x * G + h) * kD + d], fx, num);
     }
     const int64_t ph = (int64_t)(b * hq + g * G + h) * w.max_splits + split;
     if (WITH_V) w.part_o[ph * kD + d] = num / den;
-    if (d == 0) w.part_lse[ph] = Mb + log2f(den);
+    if (d == 0) w.part_lse[ph] = M * sl2 + log2f(den);
   }
+}
+
+template <typename T, int G, bool WITH_V, int MODE, bool LOGITS>
+static void launch_one(const void* q, const RowList& rows, int hq, int hkv, int batch, float scale,
+                       const AttnWorkspace& w, hipStream_t stream) {
+  auto kern = attn_stage1_mfma<T, G, WITH_V, MODE, LOGITS>;
+  const size_t lds_bytes =
+      (stage1_lds_floats<G>(WITH_V) + (LOGITS ? G * w.split_rows : 0)) * sizeof(float);
+  static size_t configured = 0;
+  if (lds_bytes > configured) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    configured = lds_bytes;
+  }
+  dim3 grid(hkv, w.max_splits, batch);  // kv head fastest: co-resident blocks cover whole token rows
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds_bytes, stream, (const T*)q, rows, hq, scale, w);
 }
 
 template <typename T, int G>
 static void launch_g(const void* q, const RowList& rows, int hq, int hkv, int batch, float scale,
                      const AttnWorkspace& w, bool with_v, bool write_logits, hipStream_t stream) {
-  dim3 grid(hkv, w.max_splits, batch);  // kv head fastest: co-resident blocks cover whole token rows
-  const bool simple = !rows.idx && !rows.page_table && rows.max_tail_len == 0 && !rows.tail_lens;
-#define OKV_LAUNCH(WV, SI)                                                                    \
-  hipLaunchKernelGGL((attn_stage1_mfma<T, G, WV, SI>), grid, dim3(256), 0, stream, (const T*)q, \
-                     rows, hq, scale, w, (int)write_logits)
-  if (with_v) {
-    if (simple) OKV_LAUNCH(true, true);
-    else OKV_LAUNCH(true, false);
-  } else {
-    if (simple) OKV_LAUNCH(false, true);
-    else OKV_LAUNCH(false, false);
-  }
-#undef OKV_LAUNCH
+  const bool no_tail = rows.max_tail_len == 0 && !rows.tail_lens;
+  int mode = 2;
+  if (!rows.idx && !rows.page_table && no_tail) mode = 0;
+  else if (rows.idx && !rows.page_table && !rows.main_lens && rows.max_main_len >= 1) mode = 1;
+#define OKV_MODES(WV, LG)                                                                  \
+  do {                                                                                     \
+    if (mode == 0) launch_one<T, G, WV, 0, LG>(q, rows, hq, hkv, batch, scale, w, stream); \
+    else if (mode == 1) launch_one<T, G, WV, 1, LG>(q, rows, hq, hkv, batch, scale, w, stream); \
+    else launch_one<T, G, WV, 2, LG>(q, rows, hq, hkv, batch, scale, w, stream);           \
+  } while (0)
+  if (!with_v) OKV_MODES(false, true);  // scoring only
+  else if (write_logits) OKV_MODES(true, true);
+  else OKV_MODES(true, false);
+#undef OKV_MODES
 }
 
 template <typename T>
@@ -300,6 +395,10 @@ static bool launch_t(const void* q, const RowList& rows, int hq, int hkv, int ba
 bool launch_stage1_mfma(int dtype, const void* q, const RowList& rows, int hq, int hkv, int batch,
                         float scale, const AttnWorkspace& w, bool with_v, bool write_logits,
                         hipStream_t stream) {
+  // token strides are used as 32-bit multipliers
+  if (rows.token_stride >= (1ll << 31) || rows.tail_token_stride >= (1ll << 31)) return false;
+  // the split's logits are staged in LDS next to the merge buffers
+  if (write_logits && (size_t)(hq / hkv) * w.split_rows * sizeof(float) > 64 * 1024) return false;
   if (dtype == OKV_BF16)
     return launch_t<BF16>(q, rows, hq, hkv, batch, scale, w, with_v, write_logits, stream);
   if (dtype == OKV_F16)

@@ -1,0 +1,119 @@
+"""Single-op timing of the HIP kernels at benchmark shapes, for profiling.
+
+    python -m omnikv_amd.microbench --op sparse --ctx 131072 --reps 50
+
+Runs `--op` back to back over `--layers` rotating K/V buffers (so no launch reads
+what the previous one left in cache), times the whole run with events on the
+launch stream and prints one JSON line with the average microseconds per call and
+the algorithmic GB/s.  Meant to sit behind `rocprofv3 --kernel-trace --stats` or
+`--pmc`: every kernel of the run belongs to the one op.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+
+import torch
+
+from . import ops, synth
+from ._lib import check, lib
+
+HQ, HKV, D = 32, 8, 128
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--op", required=True,
+                    choices=["dense", "fused", "score", "topk", "sparse", "sparse_packed", "gather", "copy"])
+    ap.add_argument("--ctx", type=int, default=131072)
+    ap.add_argument("--ratio", type=float, default=0.067)
+    ap.add_argument("--tail", type=int, default=1)
+    ap.add_argument("--layers", type=int, default=6)
+    ap.add_argument("--reps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--selector", default="softmax_sum_last")
+    ap.add_argument("--layout", default="token_major", choices=["token_major", "hf"])
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32"])
+    ap.add_argument("--split-rows", type=int, default=0)
+    ap.add_argument("--attn-variant", type=int, default=0)
+    args = ap.parse_args()
+
+    check(lib().okv_set_option(b"split_rows", args.split_rows))
+    check(lib().okv_set_option(b"attn_variant", args.attn_variant))
+    dev = torch.device("cuda:0")
+    dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[args.dtype]
+    es = 4 if dtype == torch.float32 else 2
+    n, tail, nl = args.ctx, args.tail, args.layers
+    k_sel = int(args.ratio * n)
+    gen = torch.Generator(device=dev).manual_seed(7)
+    ks, vs, qs = [], [], []
+    for _ in range(nl):
+        shape = (1, n + tail, HKV, D) if args.layout == "token_major" else (1, HKV, n + tail, D)
+        kb = torch.empty(shape, dtype=dtype, device=dev).normal_(generator=gen)
+        vb = torch.empty(shape, dtype=dtype, device=dev).normal_(generator=gen)
+        if args.layout == "token_major":
+            kb, vb = kb.permute(0, 2, 1, 3), vb.permute(0, 2, 1, 3)
+        ks.append(kb)
+        vs.append(vb)
+        qs.append(torch.randn((1, HQ, 1, D), generator=gen, device=dev).to(dtype))
+    # scores with the benchmark's distribution, and their selection
+    q0, k0, _ = synth.filter_layer_inputs(n, HQ, HKV, D)
+    ks[0][:, :, :n].copy_(k0.to(dtype))
+    qs[0] = q0.to(dtype).to(dev)
+    del k0
+    scores = ops.score(qs[0], ks[0][:, :, :n], selector=args.selector)
+    idx = ops.topk(scores, k_sel)
+    packed = [(ops.gather_rows(ks[l][:, :, :n], idx), ops.gather_rows(vs[l][:, :, :n], idx)) for l in range(nl)] \
+        if args.op == "sparse_packed" else None
+    dst = torch.empty_like(ks[0]) if args.op == "copy" else None
+
+    def call(i):
+        l = i % nl
+        if args.op == "dense":
+            return ops.dense_attn(qs[l], ks[l], vs[l])
+        if args.op == "fused":
+            return ops.dense_attn(qs[l], ks[l], vs[l], selector=args.selector, score_len=n)
+        if args.op == "score":
+            return ops.score(qs[l], ks[l][:, :, :n], selector=args.selector)
+        if args.op == "topk":
+            return ops.topk(scores, k_sel)
+        if args.op == "sparse":
+            return ops.sparse_attn(qs[l], ks[l][:, :, :n], vs[l][:, :, :n], idx=idx,
+                                   tail_k=ks[l][:, :, n:], tail_v=vs[l][:, :, n:])
+        if args.op == "sparse_packed":
+            return ops.sparse_attn(qs[l], packed[l][0], packed[l][1],
+                                   tail_k=ks[l][:, :, n:], tail_v=vs[l][:, :, n:])
+        if args.op == "gather":
+            return ops.gather_rows(ks[l][:, :, :n], idx)
+        if args.op == "copy":
+            return dst.copy_(ks[l])
+
+    row = HKV * D * es
+    algo = {
+        "dense": 2.0 * (n + tail) * row,
+        "fused": 2.0 * (n + tail) * row + 4.0 * n,
+        "score": 1.0 * n * row + 4.0 * n,
+        "topk": 4.0 * n + 4.0 * k_sel,
+        "sparse": 2.0 * (k_sel + tail) * row + 4.0 * k_sel,
+        "sparse_packed": 2.0 * (k_sel + tail) * row,
+        "gather": 2.0 * k_sel * row + 4.0 * k_sel,
+        "copy": 2.0 * (n + tail) * row,
+    }[args.op]
+    stream = torch.cuda.current_stream()
+    for i in range(args.warmup):
+        call(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for i in range(args.reps):
+        call(i)
+    e1.record(stream)
+    e1.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / args.reps
+    print(json.dumps({"op": args.op, "ctx": n, "selected": k_sel, "tail": tail, "dtype": args.dtype,
+                      "layout": args.layout, "us_per_call": us, "algorithmic_bytes": algo,
+                      "algorithmic_GBps": algo / us / 1e3, "frac_of_8TBps": algo / us / 1e3 / 8000.0}))
+
+
+if __name__ == "__main__":
+    main()
