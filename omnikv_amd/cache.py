@@ -1,0 +1,373 @@
+"""OmniKVMultiStageCache on MI355X: the reference's `cache_cls: multi`
+(modeling/spec_cache.py:253-385) with the same constructor, attributes and
+update / set_idx_on_gpu / from_dynamic_cache behaviour, over storage laid out for
+the HIP kernels.
+
+Storage.  Every layer owns preallocated token-major buffers (bsz, capacity, Hkv, D)
+-- one 2 KB (bf16, 8 kv heads) row per token and tensor -- and hands out
+(bsz, Hkv, L, D) strided VIEWS of them, so appending a decode token writes one row
+instead of re-allocating the layer (the reference's torch.cat, spec_cache.py:363-368)
+and a selected token is one contiguous row.  With real_offload the layers that only
+ever read selected rows keep their prompt K/V in PINNED host memory as interleaved
+(N, 2, Hkv, D) rows, so one host row carries a token's K and V.
+
+Two ways to consume it:
+  * the reference's: `update()` returns the tensors a third-party attention
+    would read (full cache, or gathered rows ++ tail), bit-identical to the
+    reference's values;
+  * the native one: `append()` + `attend()` / `attend_and_select()` run the HIP
+    attention kernels straight on the storage; the gather is fused into the sparse
+    attention, nothing is concatenated.
+"""
+from __future__ import annotations
+
+import threading
+from typing import Any, Dict, List, Optional, Tuple
+
+import torch
+
+from . import ops
+from ._lib import check, lib
+
+__all__ = ["OmniKVMultiStageCache", "get_cache_cls", "layer_schedule"]
+
+
+def layer_schedule(full_attn_layers, num_hidden_layers: int, num_wait_load_layers: int):
+    """layer -> (reads selected rows only, its filter layer, next full layer);
+    modeling/spec_cache.py:271-281."""
+    state = {}
+    full = list(full_attn_layers)
+    for lo in full:
+        hi = num_hidden_layers
+        for i in range(lo + 1, num_hidden_layers):
+            if i in full:
+                hi = i
+                break
+        for i in range(lo, min(hi, lo + num_wait_load_layers + 1)):
+            state[i] = (False, lo, hi)
+        for i in range(min(hi, lo + num_wait_load_layers + 1), hi):
+            state[i] = (True, lo, hi)
+    return state
+
+
+class _Store:
+    """Token-major K and V of one layer with room to append."""
+
+    def __init__(self, bsz, capacity, hkv, d, dtype, device):
+        self.k = torch.empty((bsz, capacity, hkv, d), dtype=dtype, device=device)
+        self.v = torch.empty((bsz, capacity, hkv, d), dtype=dtype, device=device)
+        self.len = 0
+
+    @property
+    def capacity(self):
+        return self.k.shape[1]
+
+    def reserve(self, n):
+        if n <= self.capacity:
+            return
+        cap = max(n, int(self.capacity * 1.5) + 64)
+        for name in ("k", "v"):
+            old = getattr(self, name)
+            new = torch.empty((old.shape[0], cap) + tuple(old.shape[2:]), dtype=old.dtype, device=old.device)
+            new[:, : self.len].copy_(old[:, : self.len])
+            setattr(self, name, new)
+
+    def append(self, key_states, value_states):
+        """key_states / value_states: (bsz, Hkv, n, D)."""
+        n = key_states.shape[2]
+        self.reserve(self.len + n)
+        self.k[:, self.len: self.len + n].copy_(key_states.permute(0, 2, 1, 3))
+        self.v[:, self.len: self.len + n].copy_(value_states.permute(0, 2, 1, 3))
+        self.len += n
+
+    def views(self, lo=0, hi=None):
+        hi = self.len if hi is None else hi
+        return self.k[:, lo:hi].permute(0, 2, 1, 3), self.v[:, lo:hi].permute(0, 2, 1, 3)
+
+
+class OmniKVMultiStageCache:
+    """Drop-in for the reference class of the same name (default DenseMore=True)."""
+
+    def __init__(self, full_attn_layers: List, num_hidden_layers, num_wait_load_layers=2, real_offload=True,
+                 max_new_tokens: int = 1024, offload_mode: str = "memcpy", cpu_num_threads: int = 8):
+        self.stage = "prefill"
+        self.full_attn_layers = full_attn_layers
+        self.num_hidden_layers = num_hidden_layers
+        self.num_wait_layers = num_wait_load_layers
+        self.layer_state = layer_schedule(full_attn_layers, num_hidden_layers, num_wait_load_layers)
+        self.need_cat_layers = []
+        self.device = "cpu" if real_offload else None
+        self.real_offload = bool(real_offload)
+        if offload_mode not in ("memcpy", "zero_copy"):
+            raise ValueError("offload_mode must be 'memcpy' or 'zero_copy'")
+        self.offload_mode = offload_mode
+        self.cpu_num_threads = int(cpu_num_threads)
+        self.max_new_tokens = int(max_new_tokens)
+        self._seen_tokens = 0
+        # reference-visible containers
+        self.key_cache: List[torch.Tensor] = []
+        self.value_cache: List[torch.Tensor] = []
+        self.part_key: Dict[int, torch.Tensor] = {}
+        self.part_value: Dict[int, torch.Tensor] = {}
+        self.tail_k: Dict[int, torch.Tensor] = {}
+        self.tail_v: Dict[int, torch.Tensor] = {}
+        # storage behind them
+        self._store: Dict[int, _Store] = {}        # GPU token-major K/V (all layers unless offloaded)
+        self._host_kv: Dict[int, torch.Tensor] = {}  # pinned (N, 2, Hkv, D) of offloaded layers
+        self._tail: Dict[int, _Store] = {}
+        self._idx: Dict[int, torch.Tensor] = {}    # filter layer -> (bsz, k) int32 on the GPU
+        self._part: Dict[int, torch.Tensor] = {}   # sparse layer -> (bsz, k, 2, Hkv, D) staged rows
+        self._part_src: Dict[int, int] = {}        # sparse layer -> id of the idx it was gathered with
+        self._staging: Dict[int, torch.Tensor] = {}
+        self._events: Dict[int, torch.cuda.Event] = {}
+        self._recorded: Dict[int, threading.Event] = {}
+        self._copy_stream: Optional[torch.cuda.Stream] = None
+        self._worker: Optional[threading.Thread] = None
+        self._prefill_len: Optional[int] = None
+
+    # ------------------------------------------------------------ storage
+    def _gpu_store(self, layer_idx, like: torch.Tensor, n_first: int) -> _Store:
+        st = self._store.get(layer_idx)
+        if st is None:
+            b, hkv, _, d = like.shape
+            st = _Store(b, n_first + self.max_new_tokens, hkv, d, like.dtype, like.device)
+            self._store[layer_idx] = st
+        return st
+
+    def _sync_lists(self, layer_idx):
+        """Keep key_cache / value_cache (the reference's public lists) pointing at views."""
+        while len(self.key_cache) <= layer_idx:
+            self.key_cache.append(None)
+            self.value_cache.append(None)
+        if layer_idx in self._host_kv:
+            h = self._host_kv[layer_idx]
+            self.key_cache[layer_idx] = h[:, 0].permute(1, 0, 2)[None]
+            self.value_cache[layer_idx] = h[:, 1].permute(1, 0, 2)[None]
+        else:
+            self.key_cache[layer_idx], self.value_cache[layer_idx] = self._store[layer_idx].views()
+
+    def get_seq_length(self, layer_idx: int = 0) -> int:
+        return self._seen_tokens
+
+    # ------------------------------------------------------------ reference API
+    def append(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int) -> None:
+        """Store the new rows of `layer_idx` (what update() does before it returns;
+        modeling/spec_cache.py:308-369)."""
+        if layer_idx == 0:
+            self._seen_tokens += key_states.shape[-2]
+        sparse = self.layer_state[layer_idx][0]
+        if sparse and self.stage != "prefill":
+            tl = self._tail.get(layer_idx)
+            if tl is None:
+                b, hkv, _, d = key_states.shape
+                tl = _Store(b, self.max_new_tokens, hkv, d, key_states.dtype, key_states.device)
+                self._tail[layer_idx] = tl
+            tl.append(key_states, value_states)
+            self.tail_k[layer_idx], self.tail_v[layer_idx] = tl.views()
+            return
+        if sparse and self.real_offload:
+            # prompt K/V of a selected-rows-only layer go to pinned host memory
+            if key_states.shape[0] != 1:
+                raise NotImplementedError("real_offload keeps one request (the reference is bs=1 too)")
+            n = key_states.shape[2]
+            host = self._host_kv.get(layer_idx)
+            if host is None:
+                hkv, d = key_states.shape[1], key_states.shape[3]
+                host = torch.empty((n, 2, hkv, d), dtype=key_states.dtype, pin_memory=True)
+                self._host_kv[layer_idx] = host
+            elif host.shape[0] != n:
+                raise NotImplementedError("an offloaded layer takes its prompt in one prefill call")
+            is_last = layer_idx == self.num_hidden_layers - 1
+            host[:, 0].copy_(key_states[0].permute(1, 0, 2), non_blocking=not is_last)
+            host[:, 1].copy_(value_states[0].permute(1, 0, 2), non_blocking=not is_last)
+            self._sync_lists(layer_idx)
+            return
+        st = self._gpu_store(layer_idx, key_states, key_states.shape[2])
+        st.append(key_states, value_states)
+        self._sync_lists(layer_idx)
+
+    def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int,
+               cache_kwargs: Optional[Dict[str, Any]] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+        """modeling/spec_cache.py:308-369: store the new rows and return what this
+        layer's attention reads."""
+        self.append(key_states, value_states, layer_idx)
+        if self.layer_state[layer_idx][0]:
+            if self.stage == "prefill":
+                return key_states, value_states
+            pk, pv = self._materialised_part(layer_idx)
+            return (torch.cat([pk, self.tail_k[layer_idx]], dim=-2),
+                    torch.cat([pv, self.tail_v[layer_idx]], dim=-2))
+        return self.key_cache[layer_idx], self.value_cache[layer_idx]
+
+    def set_idx_on_gpu(self, idx: torch.Tensor, sel_layer_idx: int) -> None:
+        """modeling/spec_cache.py:290-306.  idx: (bsz, k) ascending token indices
+        (int64 as the reference's selector returns them, or int32)."""
+        if idx.dim() == 1:
+            idx = idx[None]
+        idx32 = idx if idx.dtype == torch.int32 else idx.to(torch.int32)
+        idx32 = idx32.contiguous()
+        self._idx[sel_layer_idx] = idx32
+        hi = self.layer_state[sel_layer_idx][2]
+        lo = sel_layer_idx + self.num_wait_layers + 1
+        for i in range(lo, hi):
+            self.part_key.pop(i, None)
+            self.part_value.pop(i, None)
+            self._part_src.pop(i, None)
+        if self.real_offload and lo < hi:
+            self._start_offload(idx32, list(range(lo, hi)))
+
+    @staticmethod
+    def from_dynamic_cache(cache, full_attn_layers: List, num_hidden_layers, num_wait_load_layers=2,
+                           real_offload=True, **kwargs):
+        """modeling/spec_cache.py:371-385; `cache` is anything with key_cache /
+        value_cache lists (or transformers >= 4.54 `.layers[i].keys/.values`)."""
+        c = OmniKVMultiStageCache(full_attn_layers, num_hidden_layers, num_wait_load_layers, real_offload, **kwargs)
+        keys = getattr(cache, "key_cache", None)
+        vals = getattr(cache, "value_cache", None)
+        if keys is None and hasattr(cache, "layers"):
+            keys = [l.keys for l in cache.layers if getattr(l, "keys", None) is not None]
+            vals = [l.values for l in cache.layers if getattr(l, "values", None) is not None]
+        seen = getattr(cache, "_seen_tokens", None)
+        for i, (k, v) in enumerate(zip(keys or [], vals or [])):
+            c.append(k, v, i)
+        c._seen_tokens = seen if seen is not None else (keys[0].shape[-2] if keys else 0)
+        return c
+
+    # ------------------------------------------------------------ offload tier
+    def _start_offload(self, idx32: torch.Tensor, layers: List[int]) -> None:
+        if idx32.shape[0] != 1:
+            raise NotImplementedError("real_offload keeps one request")
+        self._join_worker()
+        dev = idx32.device
+        if self._copy_stream is None:
+            self._copy_stream = torch.cuda.Stream(device=dev)
+        k = idx32.shape[1]
+        for i in layers:
+            host = self._host_kv[i]
+            part = self._part.get(i)
+            if part is None or part.shape[1] != k:
+                self._part[i] = torch.empty((1, k) + tuple(host.shape[1:]), dtype=host.dtype, device=dev)
+            self._recorded[i] = threading.Event()
+            if i not in self._events:
+                self._events[i] = torch.cuda.Event()
+        if self.offload_mode == "zero_copy":
+            # the GPU reads the pinned rows itself: one gather per layer on the copy stream
+            self._copy_stream.wait_stream(torch.cuda.current_stream(dev))
+            with torch.cuda.stream(self._copy_stream):
+                for i in layers:
+                    host = self._host_kv[i]
+                    src = host.view(1, host.shape[0], 1, -1).permute(0, 2, 1, 3)  # (1, 1, N, 2*Hkv*D) rows
+                    dst = self._part[i].view(1, k, 1, -1).permute(0, 2, 1, 3)
+                    _gather_wide(src, idx32, dst)
+                    self._events[i].record(self._copy_stream)
+                    self._recorded[i].set()
+            return
+        host_idx = idx32[0].cpu()  # synchronises with the selection, as the reference's idx.cpu()
+        copy_stream = self._copy_stream
+
+        def work():
+            for i in layers:
+                host = self._host_kv[i]
+                row_bytes = host.stride(0) * host.element_size()
+                stg = self._staging.get(i)
+                if stg is None or stg.numel() < k * row_bytes:
+                    stg = torch.empty(k * row_bytes, dtype=torch.uint8, pin_memory=True)
+                    self._staging[i] = stg
+                else:
+                    self._events[i].synchronize()  # last step's copy out of this staging is done
+                check(lib().okv_offload_stage(
+                    host.data_ptr(), row_bytes, host_idx.data_ptr(), k, stg.data_ptr(), self.cpu_num_threads,
+                    self._part[i].data_ptr(), copy_stream.cuda_stream, None))
+                self._events[i].record(copy_stream)
+                self._recorded[i].set()
+
+        self._worker = threading.Thread(target=work, daemon=True)
+        self._worker.start()
+
+    def _join_worker(self):
+        if self._worker is not None:
+            self._worker.join()
+            self._worker = None
+
+    def _wait_part(self, layer_idx: int) -> torch.Tensor:
+        """Staged rows of an offloaded layer, ordered behind their copy on the current stream."""
+        self._recorded[layer_idx].wait()
+        torch.cuda.current_stream(self._part[layer_idx].device).wait_event(self._events[layer_idx])
+        return self._part[layer_idx]
+
+    # ------------------------------------------------------------ gathered views
+    def _materialised_part(self, layer_idx: int):
+        """(bsz, Hkv, k, D) K and V rows of the current selection; gathers on first use."""
+        sel = self.layer_state[layer_idx][1]
+        idx32 = self._idx[sel]
+        if self._part_src.get(layer_idx) != id(idx32):
+            if self.real_offload:
+                part = self._wait_part(layer_idx)
+                pk = part[:, :, 0].permute(0, 2, 1, 3)
+                pv = part[:, :, 1].permute(0, 2, 1, 3)
+            else:
+                kview, vview = self._store[layer_idx].views(0, self._prefill_rows(layer_idx))
+                pk = ops.gather_rows(kview, idx32)
+                pv = ops.gather_rows(vview, idx32)
+            self.part_key[layer_idx], self.part_value[layer_idx] = pk, pv
+            self._part_src[layer_idx] = id(idx32)
+        return self.part_key[layer_idx], self.part_value[layer_idx]
+
+    def _prefill_rows(self, layer_idx: int) -> int:
+        return self._store[layer_idx].len
+
+    # ------------------------------------------------------------ native attention
+    def attend(self, query_states: torch.Tensor, layer_idx: int, scale: Optional[float] = None) -> torch.Tensor:
+        """Decode attention of `layer_idx` over what update() would have returned,
+        without building it.  query_states: (bsz, Hq, 1, D); returns (bsz, Hq, D)."""
+        if self.layer_state[layer_idx][0] and self.stage != "prefill":
+            sel = self.layer_state[layer_idx][1]
+            tk = self.tail_k.get(layer_idx)
+            tv = self.tail_v.get(layer_idx)
+            if self.real_offload:
+                part = self._wait_part(layer_idx)
+                pk = part[:, :, 0].permute(0, 2, 1, 3)
+                pv = part[:, :, 1].permute(0, 2, 1, 3)
+                return ops.sparse_attn(query_states, pk, pv, tail_k=tk, tail_v=tv, scale=scale)
+            kview, vview = self._store[layer_idx].views()
+            return ops.sparse_attn(query_states, kview, vview, idx=self._idx[sel], tail_k=tk, tail_v=tv, scale=scale)
+        kview, vview = self._store[layer_idx].views()
+        return ops.dense_attn(query_states, kview, vview, scale=scale)
+
+    def attend_and_select(self, query_states: torch.Tensor, layer_idx: int, num_selected_tokens: int,
+                          consider_len: int, selector_cls: str = "last", scale: Optional[float] = None):
+        """Filter layer: dense attention and the filter-layer scores in one pass over
+        K, then top-k and set_idx_on_gpu (modeling/omnikv.py:189-212 followed by the
+        layer's own attention).  Returns (attention output, idx int32 (bsz, k))."""
+        kview, vview = self._store[layer_idx].views()
+        out, scores = ops.dense_attn(query_states, kview, vview, selector=selector_cls, score_len=consider_len,
+                                     scale=scale)
+        idx = ops.topk(scores, min(num_selected_tokens, consider_len))
+        self.set_idx_on_gpu(idx, layer_idx)
+        return out, idx
+
+
+def _gather_wide(src: torch.Tensor, idx32: torch.Tensor, dst: torch.Tensor) -> None:
+    """Row gather with one 'head' as wide as the whole interleaved K|V row."""
+    import ctypes as C
+
+    from ._lib import KVLayout
+
+    width = src.shape[-1]
+    if width % 128:
+        raise ValueError("row width must be a multiple of 128 elements")
+    # present each row as (width/128) heads of 128 elements
+    heads = width // 128
+    lay = KVLayout(ops._DTYPES[src.dtype], heads, heads, 128, src.stride(2), 128, 0, None, 0, 0, 0)
+    check(lib().okv_gather_rows(src.data_ptr(), C.byref(lay), idx32.data_ptr(), idx32.stride(0), None,
+                                idx32.shape[1], 1, dst.data_ptr(), dst.stride(2), 128, 0,
+                                torch.cuda.current_stream(idx32.device).cuda_stream))
+
+
+def get_cache_cls(config):
+    """modeling/spec_cache.py:829-837, restricted to the class this build provides."""
+    name2cls = {"multi": OmniKVMultiStageCache}
+    name = config.get("cache_cls", "default")
+    if name not in name2cls:
+        raise NotImplementedError(f"cache_cls={name!r}: only 'multi' is built here")
+    return name2cls[name]

@@ -1,0 +1,210 @@
+"""GPU parity of the host-side mirror of the reference interface: the multi-stage
+cache (update / set_idx_on_gpu / attend, with and without the host offload tier),
+the selector with the reference's signature, and the committed golden vectors."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from omnikv_amd import ops, selector, synth
+from omnikv_amd.cache import OmniKVMultiStageCache
+from omnikv_amd.config import OmniKVConfig
+from oracle import okv_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+TOL = {torch.float32: 1e-4, torch.bfloat16: 2e-2}
+
+
+# ------------------------------------------------------------------ golden vectors
+@pytest.mark.parametrize("n,tail", [(64, 0), (1000, 3), (4096, 1)])
+def test_kernels_against_golden(n, tail):
+    z = np.load(os.path.join(GOLDEN, f"filter_op_n{n}.npz"))
+    kk = int(z["k"])
+    q, k, v = synth.filter_layer_inputs(n)
+    _, k2, v2 = synth.filter_layer_inputs(n, seed=synth.SEED_DATA + 100)
+    qn = synth.fresh_q()
+    g = torch.Generator().manual_seed(4242 + n)
+    tk = torch.randn((1, 8, tail, 128), generator=g)
+    tv = torch.randn((1, 8, tail, 128), generator=g)
+    dense = ops.dense_attn(q.to(DEV), k.to(DEV), v.to(DEV)).cpu()
+    assert np.abs(dense[0].numpy() - z["dense_out"]).max() < 1e-4
+    for sel in ("last", "softmax_before_last", "softmax_sum_last"):
+        want_scores = torch.from_numpy(z[f"scores_{sel}"])[None]
+        want_idx = torch.from_numpy(z[f"idx_{sel}"])[None]
+        got_scores = ops.score(q.to(DEV), k.to(DEV), selector=sel).cpu()
+        assert float((got_scores - want_scores).abs().max() / want_scores.abs().max()) < 1e-4
+        # bit-exact indices on identical fp32 scores
+        assert torch.equal(ops.topk(want_scores.to(DEV), kk).cpu(), want_idx)
+        out = ops.sparse_attn(qn.to(DEV), k2.to(DEV), v2.to(DEV), idx=want_idx.to(DEV),
+                              tail_k=tk.to(DEV) if tail else None, tail_v=tv.to(DEV) if tail else None).cpu()
+        assert np.abs(out[0].numpy() - z[f"sparse_out_{sel}"]).max() < 1e-4
+
+
+def test_topk_against_golden_ties():
+    z = np.load(os.path.join(GOLDEN, "topk_ties.npz"))
+    s = torch.from_numpy(z["scores"]).to(DEV)
+    for k in z["ks"]:
+        assert np.array_equal(ops.topk(s, int(k)).cpu().numpy(), z[f"idx_k{int(k)}"])
+
+
+# ------------------------------------------------------------------ cache vs oracle cache
+def _run_decode(dtype, real_offload, offload_mode, n=777, steps=3, L=8, sel_layers=(1, 4), wait=1, ratio=0.1):
+    hq, hkv, d = 32, 8, 128
+    g = torch.Generator().manual_seed(n + L)
+    full = orc.full_attn_layers_from_select_layers(list(sel_layers), L)
+    ref = orc.OracleMultiStageCache(full, L, wait, real_offload)
+    dut = OmniKVMultiStageCache(full, L, wait, real_offload, max_new_tokens=16, offload_mode=offload_mode,
+                                cpu_num_threads=2)
+    kk = orc.num_selected_tokens(ratio, n)
+    # prefill
+    for i in range(L):
+        k = torch.randn((1, hkv, n, d), generator=g).to(dtype)
+        v = torch.randn((1, hkv, n, d), generator=g).to(dtype)
+        rk, rv = ref.update(k, v, i)
+        dk, dv = dut.update(k.to(DEV), v.to(DEV), i)
+        assert torch.equal(dk.cpu(), rk) and torch.equal(dv.cpu(), rv)
+    assert dut._seen_tokens == ref._seen_tokens == n
+    ref.stage = dut.stage = "decoding"
+    for step in range(steps):
+        for i in range(L):
+            q = torch.randn((1, hq, 1, d), generator=g).to(dtype)
+            k = torch.randn((1, hkv, 1, d), generator=g).to(dtype)
+            v = torch.randn((1, hkv, 1, d), generator=g).to(dtype)
+            if i in sel_layers:
+                # the reference selects before the layer's own update (omnikv.py:189-212)
+                scores = orc.score_tokens(q.float(), ref.key_cache[i].float(), n, "last")
+                idx = orc.select_topk(scores, kk)
+                ref.set_idx_on_gpu(idx, i)
+                got = selector.select_from_query(q.to(DEV), dut.key_cache[i], kk, n, "last")
+                assert got.dtype == torch.int64 and got.shape == idx.shape
+                assert len(set(got.cpu()[0].tolist()) & set(idx[0].tolist())) >= kk - 1
+                dut.set_idx_on_gpu(idx.to(DEV), i)  # identical selection on both sides from here on
+            rk, rv = ref.update(k, v, i)
+            want = orc.gqa_attention(q.float(), rk.float(), rv.float())[:, :, 0]
+            # native path: append + attend
+            dut.append(k.to(DEV), v.to(DEV), i)
+            out = dut.attend(q.to(DEV), i).cpu().float()
+            assert (out - want).abs().max() < TOL[dtype], (step, i)
+        # reference-style consumption of the same state: update() must return the reference's tensors
+        if step == steps - 1:
+            for i in range(L):
+                k = torch.randn((1, hkv, 1, d), generator=g).to(dtype)
+                v = torch.randn((1, hkv, 1, d), generator=g).to(dtype)
+                rk, rv = ref.update(k, v, i)
+                dk, dv = dut.update(k.to(DEV), v.to(DEV), i)
+                assert dk.shape == rk.shape
+                assert torch.equal(dk.cpu(), rk) and torch.equal(dv.cpu(), rv), i
+    return dut
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_cache_matches_reference_semantics_on_gpu(dtype):
+    dut = _run_decode(dtype, real_offload=False, offload_mode="memcpy")
+    assert sorted(dut._host_kv) == []
+    assert dut.device is None
+
+
+@pytest.mark.parametrize("mode", ["memcpy", "zero_copy"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_cache_with_host_offload_tier(dtype, mode):
+    dut = _run_decode(dtype, real_offload=True, offload_mode=mode)
+    # layers that only ever read selected rows keep their prompt K/V in pinned host memory
+    sparse = sorted(i for i, s in dut.layer_state.items() if s[0])
+    assert sorted(dut._host_kv) == sparse and sparse
+    for i in sparse:
+        assert dut._host_kv[i].is_pinned() and not dut.key_cache[i].is_cuda
+    dut._join_worker()
+
+
+def test_offload_stage_packs_rows():
+    # the C entry point alone: pinned rows -> staging -> device, runs of consecutive indices included
+    n, row = 5000, 1024
+    host = torch.randn((n, row), generator=torch.Generator().manual_seed(1)).pin_memory()
+    idx = torch.tensor(sorted(set([0, 1, 2, 3, 77, 78, 4999] + list(range(100, 3000, 7)))), dtype=torch.int32)
+    k = idx.numel()
+    stg = torch.empty((k, row)).pin_memory()
+    dst = torch.empty((k, row), device=DEV)
+    stream = torch.cuda.Stream()
+    ev = torch.cuda.Event()
+    from omnikv_amd._lib import check, lib
+    for threads in (1, 4):
+        dst.zero_()
+        torch.cuda.synchronize()
+        check(lib().okv_offload_stage(host.data_ptr(), row * 4, idx.data_ptr(), k, stg.data_ptr(), threads,
+                                      dst.data_ptr(), stream.cuda_stream, None))
+        ev.record(stream)
+        ev.synchronize()
+        assert torch.equal(dst.cpu(), host[idx.long()])
+
+
+# ------------------------------------------------------------------ selector with the reference's signature
+class _Rotary(torch.nn.Module):
+    def __init__(self, d, theta=500000.0):
+        super().__init__()
+        self.inv = 1.0 / (theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+
+    def forward(self, x, position_ids):
+        ang = position_ids[:, :, None].float() * self.inv.to(position_ids.device)[None, None, :]
+        emb = torch.cat([ang, ang], dim=-1)
+        return emb.cos().to(x.dtype), emb.sin().to(x.dtype)
+
+
+class _Attn(torch.nn.Module):
+    def __init__(self, hidden, hq, hkv, d, layer_idx):
+        super().__init__()
+        self.q_proj = torch.nn.Linear(hidden, hq * d, bias=False)
+        self.k_proj = torch.nn.Linear(hidden, hkv * d, bias=False)
+        self.num_heads, self.head_dim, self.num_key_value_heads = hq, d, hkv
+        self.num_key_value_groups = hq // hkv
+        self.layer_idx = layer_idx
+        self.rotary_emb = _Rotary(d)
+        self.config = OmniKVConfig(pretraining_tp=1)
+
+
+@pytest.mark.parametrize("selector_cls", ["last", "softmax_before_last", "uniform", "exp"])
+def test_select_tokens_by_attn_universal(selector_cls):
+    torch.manual_seed(5)
+    hidden, hq, hkv, d, n = 256, 32, 8, 128, 2000
+    attn = _Attn(hidden, hq, hkv, d, layer_idx=0)
+    win = 1 if "last" in selector_cls else 5
+    hs = torch.randn((1, win, hidden))
+    pos = torch.tensor([[n]])
+    k = torch.randn((1, hkv, n, d))
+    kk, consider = 134, n - 7
+
+    class _C:
+        key_cache = [k.to(DEV)]
+
+    got = selector.select_tokens_by_attn_universal(attn.to(DEV), hs.to(DEV), pos.to(DEV), _C(), kk, consider, 0,
+                                                   selector_cls)
+    # the same computation with the oracle on the CPU
+    attn = attn.to("cpu")
+    qs = attn.q_proj(hs).view(1, win, hq, d).transpose(1, 2)
+    cos, sin = attn.rotary_emb(qs, pos)
+    qs, _ = selector.apply_rotary_pos_emb(qs, qs, cos, sin)
+    scores = orc.score_tokens(qs.detach(), k, consider, selector_cls)
+    want = orc.select_topk(scores, kk)
+    assert got.dtype == torch.int64 and got.shape == want.shape and got.device.type == "cuda"
+    g = got.cpu()[0]
+    assert torch.all(g[1:] > g[:-1]) and int(g.max()) < consider
+    assert len(set(g.tolist()) & set(want[0].tolist())) >= kk - 2
+
+
+def test_selector_clamps_k_and_refuses_tp():
+    k = torch.randn((1, 8, 50, 128), device=DEV)
+    q = torch.randn((1, 32, 1, 128), device=DEV)
+    idx = selector.select_from_query(q, k, 4096, 50, "last")
+    assert idx.cpu()[0].tolist() == list(range(50))  # min(k, N): everything, ascending
+    attn = _Attn(64, 32, 8, 128, 0)
+    attn.config = OmniKVConfig(pretraining_tp=2)
+
+    class _C:
+        key_cache = [k]
+
+    with pytest.raises(NotImplementedError):
+        selector.select_tokens_by_attn_universal(attn, torch.zeros((1, 1, 64)), torch.zeros((1, 1)), _C(), 4, 50)

@@ -1,0 +1,203 @@
+"""CPU-side checks: golden fixtures against the oracle, the C-ABI library's exports
+and argument validation (no kernel is launched), and the host logic that mirrors the
+reference's Python interface."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from omnikv_amd import _lib, cache as okv_cache, config as okv_config, ops, selector, synth
+from oracle import okv_oracle as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+
+# ------------------------------------------------------------------ golden vectors
+@pytest.mark.parametrize("n,tail", [(64, 0), (1000, 3), (4096, 1)])
+def test_oracle_reproduces_golden(n, tail):
+    z = np.load(os.path.join(GOLDEN, f"filter_op_n{n}.npz"))
+    kk = int(z["k"])
+    assert kk == max(1, int(0.067 * n)) and int(z["tail"]) == tail
+    q, k, v = synth.filter_layer_inputs(n)
+    _, k2, v2 = synth.filter_layer_inputs(n, seed=synth.SEED_DATA + 100)
+    qn = synth.fresh_q()
+    g = torch.Generator().manual_seed(4242 + n)
+    tk = torch.randn((1, 8, tail, 128), generator=g)
+    tv = torch.randn((1, 8, tail, 128), generator=g)
+    assert np.allclose(orc.gqa_attention(q, k, v)[0, :, 0].numpy(), z["dense_out"], atol=1e-6)
+    for sel in ("last", "softmax_before_last", "softmax_sum_last"):
+        idx, scores, out = orc.filter_layer_op(q, k, v2, k2, qn, kk, sel, tk if tail else None, tv if tail else None)
+        assert np.array_equal(idx[0].numpy().astype(np.int32), z[f"idx_{sel}"])
+        assert np.allclose(scores[0].numpy(), z[f"scores_{sel}"], rtol=1e-5, atol=1e-8)
+        assert np.allclose(out[0, :, 0].numpy(), z[f"sparse_out_{sel}"], atol=1e-6)
+        # the fixture's indices are the top-k of the fixture's scores under the stable rule too
+        s = torch.from_numpy(z[f"scores_{sel}"])[None]
+        assert np.array_equal(orc.select_topk_stable(s, kk)[0].numpy().astype(np.int32), z[f"idx_{sel}"])
+
+
+def test_golden_tie_vectors():
+    z = np.load(os.path.join(GOLDEN, "topk_ties.npz"))
+    s = torch.from_numpy(z["scores"])
+    for k in z["ks"]:
+        assert np.array_equal(orc.select_topk_stable(s, int(k)).numpy().astype(np.int32), z[f"idx_k{int(k)}"])
+
+
+def test_synthetic_inputs_are_deterministic_and_shaped():
+    q, k, v = synth.filter_layer_inputs(512)
+    q2, k2, v2 = synth.filter_layer_inputs(512)
+    assert torch.equal(q, q2) and torch.equal(k, k2) and torch.equal(v, v2)
+    assert q.shape == (1, 32, 1, 128) and k.shape == (1, 8, 512, 128)
+    # the sink: token 0's keys are 8x larger than a unit normal's
+    assert float(k[0, :, 0].std()) > 6.0 and float(k[0, :, 1:].std()) < 1.5
+    # round(2%) heavy hitters stand out in the head-max score
+    s = orc.score_tokens(q, k, 512, "last")[0]
+    assert int((s[1:] > s[1:].median() + 2.0).sum()) >= 8
+    lens = synth.ragged_lengths()
+    assert lens.shape == (16,) and int(lens.min()) >= 8192 and int(lens.max()) <= 32768
+    table, total = synth.shuffled_page_table(lens, 16)
+    used = torch.cat([table[b, : (int(l) + 15) // 16] for b, l in enumerate(lens)])
+    assert sorted(used.tolist()) == list(range(total))
+    tm = synth.token_major(k)
+    assert torch.equal(tm, k) and tm.stride(2) == 8 * 128 and tm.stride(1) == 128
+
+
+# ------------------------------------------------------------------ the library
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "omnikv_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(okv_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.lib()
+    names = _declared_symbols()
+    assert "okv_score" in names and "okv_topk" in names and "okv_sparse_attn" in names
+    assert sorted(names) == sorted(_lib.EXPORTS)
+    for name in names:
+        assert getattr(lib, name) is not None
+    assert lib.okv_version() >= 1
+    assert lib.okv_strerror(0) == b"ok"
+    assert lib.okv_strerror(-3) == b"workspace too small"
+
+
+def test_workspace_sizes_are_consistent():
+    base = ops.workspace_bytes(_lib.OKV_OP_DENSE_ATTN, 1, 32, 8, 128, 131072)
+    with_scores = ops.workspace_bytes(_lib.OKV_OP_DENSE_ATTN, 1, 32, 8, 128, 131072, with_scores=True)
+    assert with_scores >= base + 32 * 131072 * 4  # room for one fp32 logit per (head, token)
+    assert ops.workspace_bytes(_lib.OKV_OP_SCORE, 1, 32, 8, 128, 4096) >= 32 * 4096 * 4
+    small = ops.workspace_bytes(_lib.OKV_OP_SPARSE_ATTN, 1, 32, 8, 128, 274, 5)
+    big = ops.workspace_bytes(_lib.OKV_OP_SPARSE_ATTN, 16, 32, 8, 128, 2195, 64)
+    assert 0 < small < big
+    assert ops.workspace_bytes(_lib.OKV_OP_TOPK, 1, 0, 0, 0, 450000) > 0
+    out = C.c_size_t(0)
+    assert _lib.lib().okv_workspace_bytes(99, C.byref(_lib.Shape(1, 32, 8, 128, 10, 0, 0)), C.byref(out)) == -1
+    assert _lib.lib().okv_workspace_bytes(0, None, C.byref(out)) == -1
+
+
+def test_argument_validation_happens_before_any_launch():
+    """Every call below must be refused on the host (no GPU is needed or touched)."""
+    lib = _lib.lib()
+    lay = _lib.KVLayout(_lib.OKV_BF16, 32, 8, 128, 1024, 128, 0, None, 0, 0, 0)
+    fake = C.c_void_p(0x1000)  # aligned, never dereferenced
+    ws = C.c_void_p(0x2000)
+    # NULL pointers
+    assert lib.okv_topk(None, 8, None, 8, None, 2, 1, fake, 2, None, 0, None) == -1
+    assert b"NULL" in lib.okv_last_error()
+    assert lib.okv_score(None, fake, C.byref(lay), None, 8, 1, 0, 0, 1.0, fake, 8, ws, 1 << 30, None) == -1
+    # unsupported geometry / dtype
+    bad = _lib.KVLayout(_lib.OKV_BF16, 32, 8, 64, 512, 64, 0, None, 0, 0, 0)
+    assert lib.okv_score(fake, fake, C.byref(bad), None, 8, 1, 0, 0, 1.0, fake, 8, ws, 1 << 30, None) == -2
+    bad = _lib.KVLayout(7, 32, 8, 128, 1024, 128, 0, None, 0, 0, 0)
+    assert lib.okv_score(fake, fake, C.byref(bad), None, 8, 1, 0, 0, 1.0, fake, 8, ws, 1 << 30, None) == -2
+    bad = _lib.KVLayout(_lib.OKV_BF16, 24, 8, 128, 1024, 128, 0, None, 0, 0, 0)  # group of 3
+    assert lib.okv_score(fake, fake, C.byref(bad), None, 8, 1, 0, 0, 1.0, fake, 8, ws, 1 << 30, None) == -2
+    bad = _lib.KVLayout(_lib.OKV_BF16, 30, 8, 128, 1024, 128, 0, None, 0, 0, 0)  # not a multiple
+    assert lib.okv_score(fake, fake, C.byref(bad), None, 8, 1, 0, 0, 1.0, fake, 8, ws, 1 << 30, None) == -1
+    # misaligned base, odd stride
+    assert lib.okv_score(fake, C.c_void_p(0x1004), C.byref(lay), None, 8, 1, 0, 0, 1.0, fake, 8, ws, 1 << 30, None) == -1
+    bad = _lib.KVLayout(_lib.OKV_BF16, 32, 8, 128, 1020, 128, 0, None, 0, 0, 0)
+    assert lib.okv_score(fake, fake, C.byref(bad), None, 8, 1, 0, 0, 1.0, fake, 8, ws, 1 << 30, None) == -1
+    # bad enums, strides smaller than the row
+    assert lib.okv_score(fake, fake, C.byref(lay), None, 8, 1, 5, 0, 1.0, fake, 8, ws, 1 << 30, None) == -1
+    assert lib.okv_score(fake, fake, C.byref(lay), None, 8, 1, 0, 0, 1.0, fake, 4, ws, 1 << 30, None) == -1
+    assert lib.okv_topk(fake, 4, None, 8, None, 2, 1, fake, 2, None, 0, None) == -1
+    assert lib.okv_topk(fake, 8, None, 8, None, 4, 1, fake, 2, None, 0, None) == -1
+    # workspace too small / missing
+    assert lib.okv_score(fake, fake, C.byref(lay), None, 4096, 1, 0, 0, 1.0, fake, 4096, ws, 16, None) == -3
+    assert b"need" in lib.okv_last_error()
+    assert lib.okv_dense_attn(fake, fake, fake, C.byref(lay), None, 4096, 1, 1.0, fake, None, 0, 0, 0, None, 0,
+                              None, 0, None) == -1
+    # nothing to attend to, tail without pointers
+    assert lib.okv_sparse_attn(fake, fake, fake, C.byref(lay), None, 0, None, 0, None, None, 0, 0, 0, None, 0, 1,
+                               1.0, fake, ws, 1 << 30, None) == -1
+    assert lib.okv_sparse_attn(fake, fake, fake, C.byref(lay), None, 0, None, 4, None, None, 1024, 128, 0, None, 2,
+                               1, 1.0, fake, ws, 1 << 30, None) == -1
+    # offload staging arguments
+    assert lib.okv_offload_stage(None, 4096, fake, 1, fake, 1, fake, None, None) == -1
+    assert lib.okv_offload_stage(fake, 4096, fake, 1, fake, 0, fake, None, None) == -1
+    # empty work is a successful no-op
+    assert lib.okv_topk(fake, 8, None, 0, None, 2, 1, fake, 2, None, 0, None) == 0
+    assert lib.okv_score(fake, fake, C.byref(lay), None, 0, 1, 0, 0, 1.0, fake, 0, ws, 1 << 30, None) == 0
+    assert lib.okv_set_option(b"no_such_option", 1) == -1
+    assert lib.okv_set_option(b"split_rows", 100) == -1
+    assert lib.okv_set_option(b"split_rows", 0) == 0
+
+
+def test_no_cpu_fallback():
+    with pytest.raises(ValueError, match="GPU"):
+        ops.topk(torch.zeros((1, 8)), 2)
+    with pytest.raises(ValueError, match="GPU"):
+        ops.score(torch.zeros((1, 32, 1, 128)), torch.zeros((1, 8, 16, 128)))
+    with pytest.raises(ValueError, match="GPU"):
+        ops.dense_attn(torch.zeros((1, 32, 1, 128)), torch.zeros((1, 8, 16, 128)), torch.zeros((1, 8, 16, 128)))
+
+
+def test_check_raises_with_detail():
+    with pytest.raises(_lib.OmniKVLibraryError, match="invalid argument"):
+        _lib.check(_lib.lib().okv_topk(None, 8, None, 8, None, 2, 1, None, 2, None, 0, None))
+
+
+# ------------------------------------------------------------------ host mirror of the reference interface
+def test_config_get_sets_and_returns_default():
+    cfg = okv_config.OmniKVConfig(do_select_layers="2,8,18", cache_cls="multi")
+    assert cfg.get("do_select_layers") == "2,8,18"
+    assert not hasattr(cfg, "window_size")
+    assert cfg.get("window_size", 16) == 16
+    assert cfg.window_size == 16  # omnikv_config.py:15-19: the default is written back
+    assert okv_cache.get_cache_cls(cfg) is okv_cache.OmniKVMultiStageCache
+    with pytest.raises(NotImplementedError):
+        okv_cache.get_cache_cls(okv_config.OmniKVConfig(cache_cls="lazy"))
+
+
+def test_cache_schedule_matches_oracle():
+    for sel, L, wait in (([2, 8, 18], 32, 1), ([4, 19, 41], 80, 1), ([2, 8, 18], 32, 2), ([0], 4, 0)):
+        full = orc.full_attn_layers_from_select_layers(sel, L)
+        c = okv_cache.OmniKVMultiStageCache(full, L, wait, real_offload=False)
+        assert c.layer_state == orc.layer_schedule(full, L, wait)
+        assert c.stage == "prefill" and c.num_wait_layers == wait and c.device is None
+    c = okv_cache.OmniKVMultiStageCache([0, 1, 2, 8, 18, 32], 32, 1, real_offload=True)
+    assert c.device == "cpu"
+    with pytest.raises(ValueError):
+        okv_cache.OmniKVMultiStageCache([0, 4], 4, 1, offload_mode="nvme")
+
+
+def test_unknown_selector_is_refused():
+    with pytest.raises(NotImplementedError):
+        selector.select_from_query(torch.zeros((1, 32, 1, 128)), torch.zeros((1, 8, 16, 128)), 4, 16, "median")
+
+
+def test_rotary_matches_complex_rotation():
+    # rotate-half RoPE == multiplying (x[i], x[i+D/2]) as a complex number by e^{i*theta_i*pos}
+    d, pos = 8, 5
+    x = torch.randn((1, 2, 1, d), generator=torch.Generator().manual_seed(3), dtype=torch.float64)
+    inv = 1.0 / (500000.0 ** (torch.arange(0, d, 2, dtype=torch.float64) / d))
+    ang = torch.cat([pos * inv, pos * inv])
+    cos, sin = ang.cos()[None, None], ang.sin()[None, None]
+    got, _ = selector.apply_rotary_pos_emb(x, x, cos, sin)
+    z = torch.complex(x[..., : d // 2], x[..., d // 2:]) * torch.polar(torch.ones(d // 2, dtype=torch.float64), pos * inv)
+    want = torch.cat([z.real, z.imag], dim=-1)
+    assert torch.allclose(got, want, atol=1e-12)
