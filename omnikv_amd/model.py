@@ -1,0 +1,245 @@
+"""A Llama-3-shaped decoder whose decode attention and token selection run on the
+HIP kernels: the counterpart of the reference's OmniKVMulLM / OmniKVMulModel /
+OmniKVMulLayer (modeling/omnikv.py:113-394) without the transformers dependency.
+
+GEMMs, norms, RoPE and the prefill attention are PyTorch-ROCm ops; the decode path
+(filter-layer scoring + top-k, dense and sparse attention, KV tiering) goes through
+omnikv_amd.cache.OmniKVMultiStageCache.  Weights are whatever the caller loads; the
+benchmark uses seeded N(0, 0.02) initialisation.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional, Tuple
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .cache import OmniKVMultiStageCache, get_cache_cls
+from .config import OmniKVConfig
+from .selector import apply_rotary_pos_emb, select_from_query
+
+
+@dataclass
+class LlamaShape:
+    hidden_size: int = 4096
+    intermediate_size: int = 14336
+    vocab_size: int = 128256
+    num_hidden_layers: int = 32
+    num_attention_heads: int = 32
+    num_key_value_heads: int = 8
+    head_dim: int = 128
+    rope_theta: float = 500000.0
+    rms_norm_eps: float = 1e-5
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, dim: int, eps: float):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(dim))
+        self.eps = eps
+
+    def forward(self, x):
+        dt = x.dtype
+        x = x.float()
+        x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.eps)
+        return self.weight * x.to(dt)
+
+
+class RotaryEmbedding(nn.Module):
+    def __init__(self, dim: int, theta: float):
+        super().__init__()
+        self.register_buffer("inv_freq", 1.0 / (theta ** (torch.arange(0, dim, 2, dtype=torch.float32) / dim)),
+                             persistent=False)
+
+    @torch.no_grad()
+    def forward(self, x, position_ids):
+        ang = position_ids[:, :, None].float() * self.inv_freq[None, None, :].to(position_ids.device)
+        emb = torch.cat([ang, ang], dim=-1)
+        return emb.cos().to(x.dtype), emb.sin().to(x.dtype)
+
+
+class MLP(nn.Module):
+    def __init__(self, s: LlamaShape):
+        super().__init__()
+        self.gate_proj = nn.Linear(s.hidden_size, s.intermediate_size, bias=False)
+        self.up_proj = nn.Linear(s.hidden_size, s.intermediate_size, bias=False)
+        self.down_proj = nn.Linear(s.intermediate_size, s.hidden_size, bias=False)
+
+    def forward(self, x):
+        return self.down_proj(F.silu(self.gate_proj(x)) * self.up_proj(x))
+
+
+class OmniKVAttention(nn.Module):
+    """q/k/v/o projections + RoPE; the attributes select_tokens_by_attn_universal reads."""
+
+    def __init__(self, s: LlamaShape, config: OmniKVConfig, layer_idx: int):
+        super().__init__()
+        self.config = config
+        self.layer_idx = layer_idx
+        self.num_heads = s.num_attention_heads
+        self.num_key_value_heads = s.num_key_value_heads
+        self.num_key_value_groups = self.num_heads // self.num_key_value_heads
+        self.head_dim = s.head_dim
+        self.q_proj = nn.Linear(s.hidden_size, self.num_heads * self.head_dim, bias=False)
+        self.k_proj = nn.Linear(s.hidden_size, self.num_key_value_heads * self.head_dim, bias=False)
+        self.v_proj = nn.Linear(s.hidden_size, self.num_key_value_heads * self.head_dim, bias=False)
+        self.o_proj = nn.Linear(self.num_heads * self.head_dim, s.hidden_size, bias=False)
+        self.rotary_emb = RotaryEmbedding(self.head_dim, s.rope_theta)
+
+    def qkv(self, hidden_states, position_ids):
+        b, n, _ = hidden_states.shape
+        q = self.q_proj(hidden_states).view(b, n, self.num_heads, self.head_dim).transpose(1, 2)
+        k = self.k_proj(hidden_states).view(b, n, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+        v = self.v_proj(hidden_states).view(b, n, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+        cos, sin = self.rotary_emb(v, position_ids)
+        q, k = apply_rotary_pos_emb(q, k, cos, sin)
+        return q, k, v
+
+
+class OmniKVMulLayer(nn.Module):
+    """modeling/omnikv.py:113-246."""
+
+    def __init__(self, s: LlamaShape, config: OmniKVConfig, layer_idx: int):
+        super().__init__()
+        self.config = config
+        self.layer_idx = layer_idx
+        self.self_attn = OmniKVAttention(s, config, layer_idx)
+        self.mlp = MLP(s)
+        self.input_layernorm = RMSNorm(s.hidden_size, s.rms_norm_eps)
+        self.post_attention_layernorm = RMSNorm(s.hidden_size, s.rms_norm_eps)
+        self.prefill_len = None
+        self.cache_cls = get_cache_cls(config)
+        self.do_select_layers = [int(i) for i in config.get("do_select_layers").split(",")]
+        self.hidden_state_window = None
+        self.selector_cls = config.get("selector_cls", "softmax_before_last")
+        self.window_size = config.get("window_size", 16)
+        self.decode_step = 0
+
+    def forward(self, hidden_states, position_ids, past_key_value: OmniKVMultiStageCache):
+        residual = hidden_states
+        hidden_states = self.input_layernorm(hidden_states)
+        q_len = hidden_states.shape[1]
+        if q_len > 1:
+            self.prefill_len = q_len
+            if "last" not in self.selector_cls and self.layer_idx in self.do_select_layers:
+                self.hidden_state_window = hidden_states[:, -self.window_size:]
+                self.decode_step = 1
+        assert isinstance(past_key_value, self.cache_cls)
+        attn = self.self_attn
+        q, k, v = attn.qkv(hidden_states, position_ids)
+        if q_len > 1:
+            # prefill: store K/V (tiered by the cache), causal attention over the prompt
+            past_key_value.append(k, v, self.layer_idx)
+            out = F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+            out = out.transpose(1, 2).reshape(hidden_states.shape[0], q_len, -1)
+        else:
+            consider_len = self.prefill_len
+            num_selected_tokens = self.config.get("num_of_selected_tokens", 4096)
+            if isinstance(num_selected_tokens, float):
+                num_selected_tokens = int(num_selected_tokens * consider_len)
+            past_key_value.append(k, v, self.layer_idx)
+            if self.layer_idx in self.do_select_layers:
+                if not self.config.get("dense_more", False):
+                    raise ValueError("dense_more=False is not supported")
+                if "last" in self.selector_cls:
+                    # scores and this layer's attention share one pass over K
+                    o, _ = past_key_value.attend_and_select(q, self.layer_idx, num_selected_tokens, consider_len,
+                                                            self.selector_cls)
+                else:
+                    forced = max(0, self.window_size - self.decode_step)
+                    self.hidden_state_window = torch.cat([self.hidden_state_window, hidden_states], dim=1)[
+                        :, -self.window_size:]
+                    win = self.hidden_state_window
+                    # every window row is rotated with the CURRENT position (modeling/omnikv.py:34-35)
+                    wq = attn.q_proj(win).view(win.shape[0], win.shape[1], attn.num_heads, attn.head_dim).transpose(1, 2)
+                    cos, sin = attn.rotary_emb(wq, position_ids)
+                    wq, _ = apply_rotary_pos_emb(wq, wq, cos, sin)
+                    kview = past_key_value.key_cache[self.layer_idx]
+                    idx = select_from_query(wq.contiguous(), kview, max(1, num_selected_tokens - forced),
+                                            consider_len - forced, self.selector_cls)
+                    tail_idx = torch.arange(self.prefill_len - forced, self.prefill_len, device=idx.device)
+                    idx = torch.cat([idx, tail_idx[None, :].repeat(idx.shape[0], 1)], dim=1)
+                    past_key_value.set_idx_on_gpu(idx, self.layer_idx)
+                    o = past_key_value.attend(q, self.layer_idx)
+                past_key_value.stage = "decoding"
+                self.decode_step += 1
+            else:
+                o = past_key_value.attend(q, self.layer_idx)
+            out = o.reshape(hidden_states.shape[0], 1, -1)
+        hidden_states = residual + attn.o_proj(out)
+        residual = hidden_states
+        hidden_states = self.post_attention_layernorm(hidden_states)
+        hidden_states = torch.cat([self.mlp(hs) for hs in torch.split(hidden_states, 4000, dim=1)], dim=1)
+        return residual + hidden_states
+
+
+class OmniKVMulModel(nn.Module):
+    def __init__(self, s: LlamaShape, config: OmniKVConfig):
+        super().__init__()
+        self.embed_tokens = nn.Embedding(s.vocab_size, s.hidden_size)
+        self.layers = nn.ModuleList([OmniKVMulLayer(s, config, i) for i in range(s.num_hidden_layers)])
+        self.norm = RMSNorm(s.hidden_size, s.rms_norm_eps)
+
+    def forward(self, input_ids, position_ids, past_key_values):
+        h = self.embed_tokens(input_ids)
+        for layer in self.layers:
+            h = layer(h, position_ids, past_key_values)
+        return self.norm(h)
+
+
+class OmniKVMulLM(nn.Module):
+    """modeling/omnikv.py:271-394: builds the cache on first use, keeps `stage`,
+    runs the model, applies lm_head to the LAST position only, returns fp32 logits."""
+
+    def __init__(self, s: LlamaShape, config: OmniKVConfig):
+        super().__init__()
+        self.shape = s
+        self.config = config
+        self.model = OmniKVMulModel(s, config)
+        self.lm_head = nn.Linear(s.hidden_size, s.vocab_size, bias=False)
+        self.cache_cls = get_cache_cls(config)
+
+    @torch.no_grad()
+    def init_weights(self, seed: int = 0, std: float = 0.02):
+        g = torch.Generator(device=self.lm_head.weight.device).manual_seed(seed)
+        for name, p in self.named_parameters():
+            if p.dim() >= 2:
+                p.normal_(0.0, std, generator=g)
+        return self
+
+    def new_cache(self, **kwargs) -> OmniKVMultiStageCache:
+        sel = [int(i) for i in self.config.get("do_select_layers").split(",")]
+        full = list(range(0, sel[0])) + sel + [self.shape.num_hidden_layers]  # modeling/omnikv.py:322-331
+        return self.cache_cls(full, self.shape.num_hidden_layers,
+                              self.config.get("num_wait_load_layers", 2), self.config.get("real_offload", True), **kwargs)
+
+    @torch.no_grad()
+    def forward(self, input_ids, past_key_values: Optional[OmniKVMultiStageCache] = None, position_ids=None,
+                **cache_kwargs):
+        n = input_ids.shape[1]
+        if not isinstance(past_key_values, self.cache_cls):
+            past_key_values = self.new_cache(**cache_kwargs)
+        past_key_values.stage = "decoding" if n == 1 else "prefill"
+        if position_ids is None:
+            start = past_key_values.get_seq_length()
+            position_ids = torch.arange(start, start + n, device=input_ids.device)[None].expand(input_ids.shape[0], -1)
+        h = self.model(input_ids, position_ids, past_key_values)
+        logits = self.lm_head(h[:, -1:]).float()
+        return logits, past_key_values
+
+    @torch.no_grad()
+    def generate_greedy(self, input_ids, num_tokens: int, **cache_kwargs) -> Tuple[torch.Tensor, List[torch.Tensor]]:
+        """num_tokens greedy tokens after the prompt; returns (tokens, per-step fp32 logits)."""
+        cache_kwargs.setdefault("max_new_tokens", num_tokens + 1)
+        logits, cache = self.forward(input_ids, None, **cache_kwargs)
+        out, all_logits = [], [logits]
+        tok = logits[:, -1].argmax(-1, keepdim=True)
+        out.append(tok)
+        for _ in range(num_tokens - 1):
+            logits, cache = self.forward(tok, cache)
+            all_logits.append(logits)
+            tok = logits[:, -1].argmax(-1, keepdim=True)
+            out.append(tok)
+        return torch.cat(out, dim=1), all_logits
