@@ -177,7 +177,8 @@ def main():
     ap.add_argument("--ratio", type=float, default=0.067)
     ap.add_argument("--selector", default="softmax_sum_last",
                     choices=["last", "softmax_before_last", "softmax_sum_last"])
-    ap.add_argument("--layout", default="token_major", choices=["token_major", "hf"])
+    ap.add_argument("--layout", default="hf", choices=["token_major", "hf"],
+                    help="hf = (1, Hkv, N, D) as the reference stores it; token_major = (1, N, Hkv, D)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32"])
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--no-cpu-baseline", action="store_true")

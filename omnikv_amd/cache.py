@@ -3,11 +3,11 @@
 update / set_idx_on_gpu / from_dynamic_cache behaviour, over storage laid out for
 the HIP kernels.
 
-Storage.  Every layer owns preallocated token-major buffers (bsz, capacity, Hkv, D)
--- one 2 KB (bf16, 8 kv heads) row per token and tensor -- and hands out
-(bsz, Hkv, L, D) strided VIEWS of them, so appending a decode token writes one row
-instead of re-allocating the layer (the reference's torch.cat, spec_cache.py:363-368)
-and a selected token is one contiguous row.  With real_offload the layers that only
+Storage.  Every layer owns preallocated buffers in the reference's own layout,
+(bsz, Hkv, capacity, D) -- each kv head one contiguous stream of 256-byte rows, which
+is what the split pass reads fastest -- and hands out (bsz, Hkv, L, D) VIEWS of them,
+so appending a decode token writes Hkv rows instead of re-allocating the layer (the
+reference's torch.cat, spec_cache.py:363-368).  With real_offload the layers that only
 ever read selected rows keep their prompt K/V in PINNED host memory as interleaved
 (N, 2, Hkv, D) rows, so one host row carries a token's K and V.
 
@@ -51,16 +51,16 @@ def layer_schedule(full_attn_layers, num_hidden_layers: int, num_wait_load_layer
 
 
 class _Store:
-    """Token-major K and V of one layer with room to append."""
+    """K and V of one layer, (bsz, Hkv, capacity, D) with room to append."""
 
     def __init__(self, bsz, capacity, hkv, d, dtype, device):
-        self.k = torch.empty((bsz, capacity, hkv, d), dtype=dtype, device=device)
-        self.v = torch.empty((bsz, capacity, hkv, d), dtype=dtype, device=device)
+        self.k = torch.empty((bsz, hkv, capacity, d), dtype=dtype, device=device)
+        self.v = torch.empty((bsz, hkv, capacity, d), dtype=dtype, device=device)
         self.len = 0
 
     @property
     def capacity(self):
-        return self.k.shape[1]
+        return self.k.shape[2]
 
     def reserve(self, n):
         if n <= self.capacity:
@@ -68,21 +68,21 @@ class _Store:
         cap = max(n, int(self.capacity * 1.5) + 64)
         for name in ("k", "v"):
             old = getattr(self, name)
-            new = torch.empty((old.shape[0], cap) + tuple(old.shape[2:]), dtype=old.dtype, device=old.device)
-            new[:, : self.len].copy_(old[:, : self.len])
+            new = torch.empty(tuple(old.shape[:2]) + (cap, old.shape[3]), dtype=old.dtype, device=old.device)
+            new[:, :, : self.len].copy_(old[:, :, : self.len])
             setattr(self, name, new)
 
     def append(self, key_states, value_states):
         """key_states / value_states: (bsz, Hkv, n, D)."""
         n = key_states.shape[2]
         self.reserve(self.len + n)
-        self.k[:, self.len: self.len + n].copy_(key_states.permute(0, 2, 1, 3))
-        self.v[:, self.len: self.len + n].copy_(value_states.permute(0, 2, 1, 3))
+        self.k[:, :, self.len: self.len + n].copy_(key_states)
+        self.v[:, :, self.len: self.len + n].copy_(value_states)
         self.len += n
 
     def views(self, lo=0, hi=None):
         hi = self.len if hi is None else hi
-        return self.k[:, lo:hi].permute(0, 2, 1, 3), self.v[:, lo:hi].permute(0, 2, 1, 3)
+        return self.k[:, :, lo:hi], self.v[:, :, lo:hi]
 
 
 class OmniKVMultiStageCache:
@@ -112,7 +112,7 @@ class OmniKVMultiStageCache:
         self.tail_k: Dict[int, torch.Tensor] = {}
         self.tail_v: Dict[int, torch.Tensor] = {}
         # storage behind them
-        self._store: Dict[int, _Store] = {}        # GPU token-major K/V (all layers unless offloaded)
+        self._store: Dict[int, _Store] = {}        # GPU K/V (all layers unless offloaded)
         self._host_kv: Dict[int, torch.Tensor] = {}  # pinned (N, 2, Hkv, D) of offloaded layers
         self._tail: Dict[int, _Store] = {}
         self._idx: Dict[int, torch.Tensor] = {}    # filter layer -> (bsz, k) int32 on the GPU

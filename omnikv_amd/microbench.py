@@ -32,7 +32,8 @@ def main():
     ap.add_argument("--reps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--selector", default="softmax_sum_last")
-    ap.add_argument("--layout", default="token_major", choices=["token_major", "hf"])
+    ap.add_argument("--layout", default="hf", choices=["token_major", "hf"],
+                    help="hf = (1, Hkv, N, D) as the reference stores it; token_major = (1, N, Hkv, D)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32"])
     ap.add_argument("--split-rows", type=int, default=0)
     ap.add_argument("--attn-variant", type=int, default=0)
