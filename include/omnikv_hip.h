@@ -135,6 +135,10 @@ int okv_score(const void* q, const void* k_base, const okv_kv_layout_t* layout,
  * omnikv-lightllm/.../flash_decoding.py:80-83.
  * seq_lens / k_per_seg: device int32[batch] or NULL (then max_seq_len / max_k
  * apply to every request).  idx_out rows beyond k_b are left untouched.
+ * ws may be NULL: then one workgroup per request does all the work.  With a
+ * workspace of okv_workspace_bytes(OKV_OP_TOPK) bytes, vectors of 16384 scores or
+ * more are processed by many workgroups in chunked passes (the workspace needs no
+ * preparation).
  */
 int okv_topk(const float* scores, int64_t score_stride, const int32_t* seq_lens,
              int32_t max_seq_len, const int32_t* k_per_seg, int32_t max_k,

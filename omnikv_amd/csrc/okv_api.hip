@@ -99,6 +99,8 @@ int carve_attn_workspace(void* ws, size_t ws_bytes, int batch, int hq, int hkv, 
   return OKV_OK;
 }
 
+size_t topk_mb_workspace_bytes(int batch, int max_seq_len);
+
 int validate_layout(const okv_kv_layout_t* layout, const void* k_base, const void* v_base) {
   OKV_REQUIRE(layout != nullptr, OKV_ERR_INVALID, "layout is NULL");
   OKV_REQUIRE(k_base != nullptr, OKV_ERR_INVALID, "k_base is NULL");
@@ -167,7 +169,7 @@ int okv_workspace_bytes(int op, const okv_shape_t* s, size_t* out_bytes) {
                                              nullptr, nullptr);
       return OKV_OK;
     case OKV_OP_TOPK:
-      *out_bytes = 256;  // the selector keeps its state in LDS
+      *out_bytes = okv::topk_mb_workspace_bytes(s->batch, s->max_seq_len);
       return OKV_OK;
     default:
       okv::set_error("unknown op %d", op);

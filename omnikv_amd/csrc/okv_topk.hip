@@ -17,6 +17,7 @@ static constexpr int kThreads = 1024;
 static constexpr int kWaves = kThreads / 64;
 static constexpr int kBins = 2048;
 static constexpr int kCandCap = 8192;  // candidate keys held in LDS (32 KB)
+static constexpr int kMultiBlockMinLen = 16384;  // below this one workgroup per request is faster
 
 __device__ __forceinline__ uint32_t score_key(float s) {
   uint32_t u = __float_as_uint(s);
@@ -296,6 +297,11 @@ __global__ __launch_bounds__(kThreads) void topk_select(const float* __restrict_
   }
 }
 
+size_t topk_mb_workspace_bytes(int batch, int max_seq_len);
+int launch_topk_mb(const float* scores, int64_t score_stride, const int32_t* seq_lens,
+                   int32_t max_seq_len, const int32_t* k_per_seg, int32_t max_k, int32_t batch,
+                   int32_t* idx_out, int64_t idx_stride, void* ws, hipStream_t stream);
+
 }  // namespace okv
 
 using namespace okv;
@@ -304,8 +310,6 @@ extern "C" int okv_topk(const float* scores, int64_t score_stride, const int32_t
                         int32_t max_seq_len, const int32_t* k_per_seg, int32_t max_k,
                         int32_t batch, int32_t* idx_out, int64_t idx_stride, void* ws,
                         size_t ws_bytes, okv_stream_t stream) {
-  (void)ws;
-  (void)ws_bytes;
   OKV_REQUIRE(scores && idx_out, OKV_ERR_INVALID, "scores or idx_out is NULL");
   OKV_REQUIRE(batch >= 1, OKV_ERR_INVALID, "batch must be >= 1");
   OKV_REQUIRE(max_seq_len >= 0 && max_k >= 0, OKV_ERR_INVALID, "negative length");
@@ -313,6 +317,11 @@ extern "C" int okv_topk(const float* scores, int64_t score_stride, const int32_t
   int kk = max_k < max_seq_len ? max_k : max_seq_len;
   OKV_REQUIRE(idx_stride >= kk, OKV_ERR_INVALID, "idx_stride < min(max_k, max_seq_len)");
   if (max_seq_len == 0 || max_k == 0) return OKV_OK;
+  // long vectors: chunked multi-workgroup passes, if the caller brought the (zero-filled) workspace
+  if (max_seq_len >= kMultiBlockMinLen && ws != nullptr &&
+      ws_bytes >= topk_mb_workspace_bytes(batch, max_seq_len))
+    return launch_topk_mb(scores, score_stride, seq_lens, max_seq_len, k_per_seg, max_k, batch,
+                          idx_out, idx_stride, ws, (hipStream_t)stream);
   hipLaunchKernelGGL(topk_select, dim3(batch), dim3(kThreads), 0, (hipStream_t)stream, scores,
                      score_stride, seq_lens, max_seq_len, k_per_seg, max_k, idx_out, idx_stride);
   OKV_HIP_CHECK(hipGetLastError());

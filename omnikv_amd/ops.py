@@ -152,10 +152,11 @@ def topk(scores: torch.Tensor, k: int, seq_lens: Optional[torch.Tensor] = None,
         out = torch.empty((batch, kk), dtype=torch.int32, device=scores.device)
     if kk == 0:
         return out
+    ws = _workspace(scores.device, workspace_bytes(_lib.OKV_OP_TOPK, batch, 0, 0, 0, n))
     check(lib().okv_topk(
         scores.data_ptr(), scores.stride(0), _lens(seq_lens, batch, "seq_lens"), n,
         _lens(k_per_seg, batch, "k_per_seg"), k, batch, out.data_ptr(), out.stride(0),
-        None, 0, _stream_ptr(scores.device)))
+        ws.data_ptr(), ws.numel(), _stream_ptr(scores.device)))
     return out
 
 

@@ -230,3 +230,46 @@ def test_filter_layer_op_config0(selector):
     assert len(same) >= kk - 1
     if len(same) == kk:
         assert (out.cpu() - out_w[:, :, 0, :]).abs().max() < 1e-4
+
+
+# ------------------------------------------------ long vectors: the chunked multi-workgroup path
+def _topk_single_workgroup(scores_dev, k):
+    """The one-workgroup-per-request kernel, selected by passing no workspace."""
+    import ctypes as C
+
+    from omnikv_amd._lib import check, lib
+    out = torch.empty((scores_dev.shape[0], min(k, scores_dev.shape[1])), dtype=torch.int32, device=DEV)
+    check(lib().okv_topk(scores_dev.data_ptr(), scores_dev.stride(0), None, scores_dev.shape[1], None, k,
+                         scores_dev.shape[0], out.data_ptr(), out.stride(0), None, 0,
+                         torch.cuda.current_stream().cuda_stream))
+    return out
+
+
+@pytest.mark.parametrize("n", [16384, 16385, 40000, 131072 + 3])
+def test_topk_long_special_values_and_both_kernels(n):
+    g = torch.Generator().manual_seed(n)
+    s = torch.randn((2, n), generator=g)
+    s[0, 5] = float("inf"); s[0, n - 1] = float("inf"); s[0, 6] = float("-inf")
+    s[0, 100:200] = 0.0; s[0, 150:160] = -0.0
+    s[1, 7] = float("nan"); s[1, n - 2] = float("nan")
+    s[1, 4096:8192] = 1.25  # a whole chunk of one value
+    for k in (1, 2, 3, 150, n // 15, n - 1, n):
+        _check_topk(s, k)
+        sd = s.to(DEV)
+        assert torch.equal(_topk_single_workgroup(sd, k), ops.topk(sd, k))
+    z = torch.zeros((1, n))
+    assert torch.equal(ops.topk(z.to(DEV), 1000).cpu(), torch.arange(1000, dtype=torch.int32)[None])
+    # unaligned score rows (a view starting one float into a buffer)
+    buf = torch.randn((n + 1,), generator=g).to(DEV)
+    view = buf[1:][None]
+    assert torch.equal(ops.topk(view, 500).cpu().to(torch.int64), orc.select_topk_stable(view.cpu(), 500))
+
+
+def test_topk_repeated_calls_leave_workspace_clean():
+    g = torch.Generator().manual_seed(77)
+    for i in range(6):  # same workspace, different lengths and distributions each time
+        n = [131072, 20000, 450000, 16384, 70001, 131072][i]
+        s = torch.randn((1, n), generator=g) * (10.0 ** (i - 3))
+        if i % 2:
+            s = torch.softmax(s * 3, dim=-1)
+        _check_topk(s, max(1, int(0.067 * n)))
