@@ -29,6 +29,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the dense split pass from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE
+# (profiles/dense_split_pass_pmc.txt), keyed by (context, tail, dtype); None when not measured.
+TRAFFIC_BYTES = {}
 HQ, HKV, D, LAYERS = 32, 8, 128, 32
 FILTER_LAYERS = (2, 8, 18)
 WAIT = 1
@@ -243,6 +246,11 @@ def main():
 
         dense_pass()
         dense_ms = time_events(dense_pass, reps, stream) / len(dense_layers)
+        # the split pass alone (the dominant kernel), merge launch left out
+        check(lib().okv_set_option(b"skip_merge", 1))
+        dense_pass()
+        split_ms = time_events(dense_pass, reps, stream) / len(dense_layers)
+        check(lib().okv_set_option(b"skip_merge", 0))
         detail = {}
         if args.detail:
             fl = FILTER_LAYERS[0]
@@ -266,7 +274,7 @@ def main():
             print(json.dumps(detail), file=sys.stderr)
 
     dense_bytes = 2.0 * (n + tail) * HKV * D * esize  # K and V rows once each
-    achieved = dense_bytes / (dense_ms * 1e-3) / 1e9
+    achieved = dense_bytes / (split_ms * 1e-3) / 1e9
     kinds = schedule()
     step_bytes = 0.0
     for l, (kind, _) in kinds.items():
@@ -298,10 +306,12 @@ def main():
         "decode_tokens_per_s_attention_only": 1e3 / wall_ms,
         "step_hbm_gbs": step_bytes / (wall_ms * 1e-3) / 1e9,
         "roofline": {
-            "kernel": "dense split attention (stage 1 + merge), N+tail rows",
+            "kernel": "okv::attn_stage1_mfma<BF16,4,true,0,false> (dense split pass over N+tail rows of K and V)"
+            if dtype != torch.float32 else "okv::attn_stage1_generic<float,4,true> (dense split pass)",
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-            "bytes_per_launch": dense_bytes, "avg_launch_us": dense_ms * 1e3,
+            "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES.get((n, tail, args.dtype)),
+            "bytes_per_launch": dense_bytes, "avg_launch_us": split_ms * 1e3,
+            "with_merge_launch_us": dense_ms * 1e3,
         },
     }
     if not args.no_cpu_baseline:

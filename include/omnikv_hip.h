@@ -98,8 +98,9 @@ int okv_version(void);
 /* Process-wide tuning switches, for A/B measurements.  "attn_variant": 0 (default)
  * runs 16-bit attention / scoring on the matrix-core kernel, 1 forces the portable
  * VALU kernel for every dtype.  "split_rows": rows per split of the attention /
- * scoring pass, 0 = automatic.  Set options before sizing workspaces.  No reference
- * counterpart. */
+ * scoring pass, 0 = automatic.  "skip_merge": 1 launches the split pass of the
+ * attention entry points alone (outputs are then NOT produced; for timing that kernel
+ * in isolation).  Set options before sizing workspaces.  No reference counterpart. */
 int okv_set_option(const char* name, int value);
 
 /* Bytes of scratch `op` needs for `shape`.  No reference counterpart: the

@@ -47,6 +47,12 @@ static int choose_split_rows(int batch, int hkv, int total_rows, bool with_v, bo
   for (int64_t rounds = 1;; ++rounds) {
     int64_t rows = (work + rounds * capacity - 1) / (rounds * capacity);
     rows = (rows + 63) / 64 * 64;
+    if (rounds == 1 && with_v && rows <= 128) {
+      // a few thousand rows (sparse layers): the pass is a latency chain, and fewer, fatter
+      // workgroups (three tiles per wave, a third fewer partials to merge) finish sooner
+      rows = (work + capacity * 2 / 3 - 1) / (capacity * 2 / 3);
+      rows = (rows + 63) / 64 * 64;
+    }
     if (rows <= cap_rows) return (int)rows;
   }
 }

@@ -171,23 +171,35 @@ __global__ __launch_bounds__(256) void attn_merge(RowList rows, int hq, AttnWork
 
   float m = -INFINITY, den = 0.f, mA = -INFINITY, denA = 0.f;
   float4 num = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll 4
-  for (int s = sl; s < ns; s += 8) {
-    const float x = lse[s];
-    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (with_v) o = po[(int64_t)s * 32];
-    const float mn = fmaxf(m, x);
-    const float a = exp2f(m - mn), f = exp2f(x - mn);
-    den = fmaf(den, a, f);
-    num.x = fmaf(num.x, a, f * o.x);
-    num.y = fmaf(num.y, a, f * o.y);
-    num.z = fmaf(num.z, a, f * o.z);
-    num.w = fmaf(num.w, a, f * o.w);
-    m = mn;
-    if (s < nA) {
-      const float mnA = fmaxf(mA, x);
-      denA = fmaf(denA, exp2f(mA - mnA), exp2f(x - mnA));
-      mA = mnA;
+  constexpr int U = 8;  // splits in flight per thread: all loads of a batch leave before any is used
+  for (int s0 = sl; s0 < ns; s0 += 8 * U) {
+    float xs[U];
+    float4 os[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int s = s0 + 8 * u;
+      xs[u] = s < ns ? lse[s] : -INFINITY;
+      os[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (with_v && s < ns) os[u] = po[(int64_t)s * 32];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int s = s0 + 8 * u;
+      if (s >= ns) break;
+      const float x = xs[u];
+      const float mn = fmaxf(m, x);
+      const float a = exp2f(m - mn), f = exp2f(x - mn);
+      den = fmaf(den, a, f);
+      num.x = fmaf(num.x, a, f * os[u].x);
+      num.y = fmaf(num.y, a, f * os[u].y);
+      num.z = fmaf(num.z, a, f * os[u].z);
+      num.w = fmaf(num.w, a, f * os[u].w);
+      m = mn;
+      if (s < nA) {
+        const float mnA = fmaxf(mA, x);
+        denA = fmaf(denA, exp2f(mA - mnA), exp2f(x - mnA));
+        mA = mnA;
+      }
     }
   }
   snum[sl][dq] = num;
@@ -261,6 +273,7 @@ __global__ __launch_bounds__(256) void score_finish(RowList rows, int hq, AttnWo
 
 // ----------------------------------------------------------------- launch
 int g_attn_variant = 0;  // 0 = pick per dtype, 1 = portable VALU stage 1 everywhere
+int g_skip_merge = 0;    // 1 = launch the split pass alone (timing it in isolation)
 
 bool launch_stage1_mfma(int dtype, const void* q, const RowList& rows, int hq, int hkv, int batch,
                         float scale, const AttnWorkspace& w, bool with_v, bool write_logits,
@@ -298,7 +311,7 @@ static int launch_typed(const void* q, const RowList& rows, const okv_kv_layout_
     default: set_error("GQA group %d not supported", G); return OKV_ERR_UNSUPPORTED;
   }
   const bool need_score_lse = want_scores && normalise == OKV_NORM_SOFTMAX;
-  if (with_v || need_score_lse)
+  if (!g_skip_merge && (with_v || need_score_lse))
     hipLaunchKernelGGL((attn_merge<T>), dim3(hq, batch), dim3(256), 0, stream, rows, hq, w,
                        (T*)out, (int)with_v, (int)need_score_lse);
   if (want_scores && rows.max_score_len > 0)
@@ -351,6 +364,11 @@ int okv_set_option(const char* name, int value) {
   if (strcmp(name, "attn_variant") == 0) {
     OKV_REQUIRE(value == 0 || value == 1, OKV_ERR_INVALID, "attn_variant must be 0 or 1");
     g_attn_variant = value;
+    return OKV_OK;
+  }
+  if (strcmp(name, "skip_merge") == 0) {
+    OKV_REQUIRE(value == 0 || value == 1, OKV_ERR_INVALID, "skip_merge must be 0 or 1");
+    g_skip_merge = value;
     return OKV_OK;
   }
   if (strcmp(name, "split_rows") == 0) {
