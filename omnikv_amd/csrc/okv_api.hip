@@ -39,10 +39,13 @@ static int num_compute_units() {
 // every workgroup getting the same share of rows: all of them start together and
 // finish together, in one round when the split fits the row cap, else in the fewest
 // equal rounds.  The cap keeps the LDS staging of a scored split's logits small.
-static int choose_split_rows(int batch, int hkv, int total_rows, bool with_v, bool with_logits) {
+static int choose_split_rows(int batch, int hq, int hkv, int total_rows, bool with_v,
+                             bool with_logits) {
   if (g_split_rows_override > 0) return g_split_rows_override;
   const int64_t capacity = (int64_t)num_compute_units() * (with_v ? 3 : 6);
-  const int64_t cap_rows = with_logits ? 1024 : 4096;
+  // a scored split stages G*rows fp32 logits in LDS: keep that within 32 KB
+  const int group = hkv > 0 && hq >= hkv ? hq / hkv : 1;
+  const int64_t cap_rows = with_logits ? (8192 / group) / 64 * 64 : 4096;
   const int64_t work = (int64_t)(total_rows > 0 ? total_rows : 1) * hkv * (batch > 0 ? batch : 1);
   for (int64_t rounds = 1;; ++rounds) {
     int64_t rows = (work + rounds * capacity - 1) / (rounds * capacity);
@@ -61,7 +64,7 @@ size_t attn_workspace_bytes(int batch, int hq, int hkv, int d, int max_main, int
                             int max_score, bool with_v, bool with_logits, int* split_rows,
                             int* max_splits) {
   int L = max_main + max_tail;
-  int C = choose_split_rows(batch, hkv, L, with_v, with_logits);
+  int C = choose_split_rows(batch, hq, hkv, L, with_v, with_logits);
   int S = (L + C - 1) / C + (max_score > 0 ? 1 : 0);
   if (S < 1) S = 1;
   if (split_rows) *split_rows = C;

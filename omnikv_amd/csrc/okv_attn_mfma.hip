@@ -195,7 +195,7 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
     for (int d = 0; d < 8; ++d) acc[h][d] = 0.f;
   const float sl2 = scale * kLog2e;
   const bool scored = LOGITS && begin < A;  // a scored split ends at or before A
-  float* slog = lds + stage1_lds_floats<G>(WITH_V);  // [G][split_rows] scaled logits of the split
+  float* slog = lds;  // [G][split_rows] scaled logits of the split; flushed before LDS is reused below
 
   auto compute = [&](int tbase, const uint4 (&kf)[4], const uint4 (&vf)[4]) {
     f32x4_t S = {0.f, 0.f, 0.f, 0.f};
@@ -292,6 +292,26 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
     }
   }
 
+  // ---- a scored split hands its logits over, then LDS changes hands
+  if (scored) {
+    __syncthreads();
+    const int quads = w.split_rows >> 2;
+    for (int o = threadIdx.x; o < G * quads; o += 256) {
+      const int h = o / quads, r = begin + 4 * (o % quads);
+      if (r >= end) continue;
+      const float4 v = *reinterpret_cast<const float4*>(slog + h * w.split_rows + (r - begin));
+      float* lp = w.logits + (int64_t)(b * hq + g * G + h) * w.logits_stride + r;
+      if (r + 3 < end) {
+        *reinterpret_cast<float4*>(lp) = v;
+      } else {
+        lp[0] = v.x;
+        if (r + 1 < end) lp[1] = v.y;
+        if (r + 2 < end) lp[2] = v.z;
+      }
+    }
+    __syncthreads();
+  }
+
   // ---- the 16 lane rows of the block meet in LDS
   float* sm = lds;                // [16][G] running max (raw units)
   float* sl = lds + 16 * G;       // [16][G] sum of exp
@@ -310,22 +330,6 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
     }
   }
   __syncthreads();
-  if (scored) {
-    const int quads = w.split_rows >> 2;
-    for (int o = threadIdx.x; o < G * quads; o += 256) {
-      const int h = o / quads, r = begin + 4 * (o % quads);
-      if (r >= end) continue;
-      const float4 v = *reinterpret_cast<const float4*>(slog + h * w.split_rows + (r - begin));
-      float* lp = w.logits + (int64_t)(b * hq + g * G + h) * w.logits_stride + r;
-      if (r + 3 < end) {
-        *reinterpret_cast<float4*>(lp) = v;
-      } else {
-        lp[0] = v.x;
-        if (r + 1 < end) lp[1] = v.y;
-        if (r + 2 < end) lp[2] = v.z;
-      }
-    }
-  }
   for (int o = threadIdx.x; o < G * kD; o += 256) {
     const int h = o / kD, d = o % kD;
     float M = -INFINITY;
@@ -349,8 +353,9 @@ template <typename T, int G, bool WITH_V, int MODE, bool LOGITS>
 static void launch_one(const void* q, const RowList& rows, int hq, int hkv, int batch, float scale,
                        const AttnWorkspace& w, hipStream_t stream) {
   auto kern = attn_stage1_mfma<T, G, WITH_V, MODE, LOGITS>;
-  const size_t lds_bytes =
-      (stage1_lds_floats<G>(WITH_V) + (LOGITS ? G * w.split_rows : 0)) * sizeof(float);
+  size_t lds_floats = stage1_lds_floats<G>(WITH_V);  // the logits staging aliases the merge buffers
+  if (LOGITS && (size_t)G * w.split_rows > lds_floats) lds_floats = (size_t)G * w.split_rows;
+  const size_t lds_bytes = lds_floats * sizeof(float);
   static size_t configured = 0;
   if (lds_bytes > configured) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -398,7 +403,7 @@ bool launch_stage1_mfma(int dtype, const void* q, const RowList& rows, int hq, i
   // token strides are used as 32-bit multipliers
   if (rows.token_stride >= (1ll << 31) || rows.tail_token_stride >= (1ll << 31)) return false;
   // the split's logits are staged in LDS next to the merge buffers
-  if (write_logits && (size_t)(hq / hkv) * w.split_rows * sizeof(float) > 64 * 1024) return false;
+  if (write_logits && (size_t)(hq / hkv) * w.split_rows * sizeof(float) > 48 * 1024) return false;
   if (dtype == OKV_BF16)
     return launch_t<BF16>(q, rows, hq, hkv, batch, scale, w, with_v, write_logits, stream);
   if (dtype == OKV_F16)
