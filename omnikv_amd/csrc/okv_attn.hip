@@ -278,6 +278,9 @@ int g_skip_merge = 0;    // 1 = launch the split pass alone (timing it in isolat
 bool launch_stage1_mfma(int dtype, const void* q, const RowList& rows, int hq, int hkv, int batch,
                         float scale, const AttnWorkspace& w, bool with_v, bool write_logits,
                         hipStream_t stream);
+bool launch_score_raw_mfma(int dtype, const void* q, const RowList& rows, int hq, int hkv, int batch,
+                           float scale, int head_reduce, float* scores, int64_t score_stride,
+                           hipStream_t stream);
 
 template <typename T, int G>
 static void launch_stage1(const void* q, const RowList& rows, int hq, int hkv, int batch,
@@ -299,6 +302,13 @@ static int launch_typed(const void* q, const RowList& rows, const okv_kv_layout_
                         const AttnWorkspace& w, hipStream_t stream) {
   const int hq = lay->num_q_heads, hkv = lay->num_kv_heads, G = hq / hkv;
   const bool want_scores = scores != nullptr;
+  // raw scores alone need no normaliser: one launch that reduces the heads in the workgroup
+  if (g_attn_variant != 1 && !with_v && want_scores && normalise == OKV_NORM_RAW &&
+      launch_score_raw_mfma(lay->dtype, q, rows, hq, hkv, batch, scale, head_reduce, scores, score_stride,
+                            stream)) {
+    OKV_HIP_CHECK(hipGetLastError());
+    return OKV_OK;
+  }
   if (g_attn_variant != 1 &&
       launch_stage1_mfma(lay->dtype, q, rows, hq, hkv, batch, scale, w, with_v, want_scores, stream)) {
     // 16-bit K/V: stage 1 ran on the matrix-core kernel

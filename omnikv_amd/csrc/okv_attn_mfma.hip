@@ -397,6 +397,155 @@ static bool launch_t(const void* q, const RowList& rows, int hq, int hkv, int ba
   return false;
 }
 
+// ---------------------------------------------------------------------------
+// Raw (un-normalised) scores in ONE launch.  A workgroup owns a range of rows and ALL
+// kv heads, one wave per kv head: every wave streams its head's K rows through the
+// same MFMA tiles as above, reduces its G q heads with lane swaps, and leaves one
+// value per row in LDS; the workgroup then reduces over kv heads and writes the scores.
+// No logits round trip, no merge, no finishing launch.
+template <typename T, int G, bool PAGED>
+__global__ __launch_bounds__(1024) void score_raw_mfma(const T* __restrict__ q, RowList rows, int hq,
+                                                       float scale, int head_reduce,
+                                                       int rows_per_block, float* __restrict__ scores,
+                                                       int64_t score_stride) {
+  extern __shared__ float lds[];  // [kv heads][rows_per_block]
+  const int b = blockIdx.y;
+  const int A = rl_score_len(rows, b);
+  const int begin = blockIdx.x * rows_per_block;
+  const int end = min(begin + rows_per_block, A);
+  if (begin >= end) return;
+  const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int r16 = lane & 15, j4 = lane >> 4;
+  const bool is_max = head_reduce == OKV_REDUCE_MAX;
+
+  uint4 qf[4];
+  {
+    const int hcol = r16 < G ? r16 : G - 1;
+    const T* qp = q + ((int64_t)(b * hq + g * G + hcol) * kD + 8 * j4);
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const uint4 v = *reinterpret_cast<const uint4*>(qp + 32 * s);
+      qf[s] = r16 < G ? v : make_uint4(0, 0, 0, 0);
+    }
+  }
+  const T* kb = reinterpret_cast<const T*>(rows.k_base) + (int64_t)g * rows.head_stride + 8 * j4 +
+                (PAGED ? 0 : (int64_t)b * rows.batch_stride);
+  const uint32_t ts = (uint32_t)rows.token_stride;
+  const int last = end - 1;
+  auto load_tile = [&](int tbase, uint4 (&kf)[4]) {
+    int r = tbase + r16;
+    r = r < last ? r : last;
+    const T* kp;
+    if (PAGED) {
+      const int page = rows.page_table[(int64_t)b * rows.page_table_stride + r / rows.page_size];
+      kp = kb + (int64_t)page * rows.page_stride + (uint64_t)(uint32_t)(r % rows.page_size) * ts;
+    } else {
+      kp = kb + (uint64_t)(uint32_t)r * ts;
+    }
+#pragma unroll
+    for (int s = 0; s < 4; ++s) kf[s] = *reinterpret_cast<const uint4*>(kp + 32 * s);
+  };
+  float* mine = lds + g * rows_per_block;
+  auto compute = [&](int tbase, const uint4 (&kf)[4]) {
+    f32x4_t S = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 4; ++s) S = mfma16((const T*)nullptr, kf[s], qf[s], S);
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[i] = S[i] * scale;
+#pragma unroll
+      for (int o = 1; o < G; o <<= 1) {  // lanes 0..G-1 of the lane row hold the G heads
+        const float x = __shfl_xor(v[i], o);
+        v[i] = is_max ? fmaxf(v[i], x) : v[i] + x;
+      }
+    }
+    if (r16 == 0)
+      *reinterpret_cast<float4*>(mine + (tbase - begin) + 4 * j4) = make_float4(v[0], v[1], v[2], v[3]);
+  };
+  {
+    uint4 kA[4], kB[4];
+    const int t_last = begin + ((last - begin) >> 4 << 4);
+    int t = begin;
+    load_tile(t, kA);
+    if (t == t_last) {
+      compute(t, kA);
+    } else {
+      while (true) {
+        load_tile(min(t + 16, t_last), kB);
+        compute(t, kA);
+        t += 16;
+        load_tile(min(t + 16, t_last), kA);
+        compute(t, kB);
+        if (t == t_last) break;
+        t += 16;
+        if (t == t_last) {
+          compute(t, kA);
+          break;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  const int nheads = blockDim.x >> 6;
+  for (int r = threadIdx.x; r < end - begin; r += blockDim.x) {
+    float acc = lds[r];
+    for (int x = 1; x < nheads; ++x) {
+      const float y = lds[x * rows_per_block + r];
+      acc = is_max ? fmaxf(acc, y) : acc + y;
+    }
+    scores[(int64_t)b * score_stride + begin + r] = acc;
+  }
+}
+
+template <typename T, int G>
+static void launch_score_raw_g(const void* q, const RowList& rows, int hq, int hkv, int batch,
+                               float scale, int head_reduce, float* scores, int64_t score_stride,
+                               hipStream_t stream) {
+  int cus = 256, dev = 0;
+  if (hipGetDevice(&dev) == hipSuccess) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
+  }
+  // one round of workgroups, three resident per CU, equal shares of the rows
+  int64_t per = ((int64_t)rows.max_score_len * batch + (int64_t)cus * 3 - 1) / ((int64_t)cus * 3);
+  int rpb = (int)((per + 15) / 16 * 16);
+  if (rpb < 64) rpb = 64;
+  if (rpb > 1024) rpb = 1024;
+  dim3 grid((rows.max_score_len + rpb - 1) / rpb, batch), block(64 * hkv);
+  const size_t lds_bytes = (size_t)hkv * rpb * sizeof(float);
+  if (rows.page_table)
+    hipLaunchKernelGGL((score_raw_mfma<T, G, true>), grid, block, lds_bytes, stream, (const T*)q, rows, hq,
+                       scale, head_reduce, rpb, scores, score_stride);
+  else
+    hipLaunchKernelGGL((score_raw_mfma<T, G, false>), grid, block, lds_bytes, stream, (const T*)q, rows,
+                       hq, scale, head_reduce, rpb, scores, score_stride);
+}
+
+template <typename T>
+static bool launch_score_raw_t(const void* q, const RowList& rows, int hq, int hkv, int batch, float scale,
+                               int head_reduce, float* scores, int64_t score_stride, hipStream_t stream) {
+  switch (hq / hkv) {
+    case 1: launch_score_raw_g<T, 1>(q, rows, hq, hkv, batch, scale, head_reduce, scores, score_stride, stream); return true;
+    case 2: launch_score_raw_g<T, 2>(q, rows, hq, hkv, batch, scale, head_reduce, scores, score_stride, stream); return true;
+    case 4: launch_score_raw_g<T, 4>(q, rows, hq, hkv, batch, scale, head_reduce, scores, score_stride, stream); return true;
+    case 8: launch_score_raw_g<T, 8>(q, rows, hq, hkv, batch, scale, head_reduce, scores, score_stride, stream); return true;
+  }
+  return false;
+}
+
+// Stand-alone raw scoring (no V, no softmax) of 16-bit K with at most 16 kv heads.
+bool launch_score_raw_mfma(int dtype, const void* q, const RowList& rows, int hq, int hkv, int batch,
+                           float scale, int head_reduce, float* scores, int64_t score_stride,
+                           hipStream_t stream) {
+  if (hkv > 16 || rows.idx || rows.token_stride >= (1ll << 31)) return false;
+  if (dtype == OKV_BF16)
+    return launch_score_raw_t<BF16>(q, rows, hq, hkv, batch, scale, head_reduce, scores, score_stride, stream);
+  if (dtype == OKV_F16)
+    return launch_score_raw_t<F16>(q, rows, hq, hkv, batch, scale, head_reduce, scores, score_stride, stream);
+  return false;
+}
+
 bool launch_stage1_mfma(int dtype, const void* q, const RowList& rows, int hq, int hkv, int batch,
                         float scale, const AttnWorkspace& w, bool with_v, bool write_logits,
                         hipStream_t stream) {
