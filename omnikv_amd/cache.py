@@ -89,7 +89,7 @@ class OmniKVMultiStageCache:
     """Drop-in for the reference class of the same name (default DenseMore=True)."""
 
     def __init__(self, full_attn_layers: List, num_hidden_layers, num_wait_load_layers=2, real_offload=True,
-                 max_new_tokens: int = 1024, offload_mode: str = "memcpy", cpu_num_threads: int = 8):
+                 max_new_tokens: int = 1024, offload_mode: str = "zero_copy", cpu_num_threads: int = 8):
         self.stage = "prefill"
         self.full_attn_layers = full_attn_layers
         self.num_hidden_layers = num_hidden_layers

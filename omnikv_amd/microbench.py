@@ -24,7 +24,9 @@ HQ, HKV, D = 32, 8, 128
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--op", required=True,
-                    choices=["dense", "fused", "score", "topk", "sparse", "sparse_packed", "gather", "copy"])
+                    choices=["dense", "fused", "score", "topk", "sparse", "sparse_packed", "gather", "copy",
+                             "offload_memcpy", "offload_zero_copy", "h2d"])
+    ap.add_argument("--cpu-threads", type=int, default=8, help="packing threads of the offload tier")
     ap.add_argument("--ctx", type=int, default=131072)
     ap.add_argument("--ratio", type=float, default=0.067)
     ap.add_argument("--tail", type=int, default=1)
@@ -67,6 +69,20 @@ def main():
     packed = [(ops.gather_rows(ks[l][:, :, :n], idx), ops.gather_rows(vs[l][:, :, :n], idx)) for l in range(nl)] \
         if args.op == "sparse_packed" else None
     dst = torch.empty_like(ks[0]) if args.op == "copy" else None
+    off = None
+    if args.op.startswith("offload") or args.op == "h2d":
+        # one offloaded layer group: `nl` layers whose prompt K/V live in pinned host memory
+        from .cache import OmniKVMultiStageCache
+        off = OmniKVMultiStageCache([0, nl + 2], nl + 2, num_wait_load_layers=1, real_offload=True,
+                                    offload_mode="zero_copy" if args.op == "offload_zero_copy" else "memcpy",
+                                    cpu_num_threads=args.cpu_threads)
+        for l in range(nl + 2):
+            off.append(ks[l % nl][:, :, :n], vs[l % nl][:, :, :n], l)
+        torch.cuda.synchronize()
+        off.stage = "decoding"
+        if args.op == "h2d":
+            hsrc = torch.empty(k_sel * 2 * HKV * D * es, dtype=torch.uint8).pin_memory()
+            hdst = torch.empty(k_sel * 2 * HKV * D * es, dtype=torch.uint8, device=dev)
 
     def call(i):
         l = i % nl
@@ -88,6 +104,14 @@ def main():
             return ops.gather_rows(ks[l][:, :, :n], idx)
         if args.op == "copy":
             return dst.copy_(ks[l])
+        if args.op == "h2d":
+            return hdst.copy_(hsrc, non_blocking=True)
+        if off is not None:
+            # select once, stage the rows of all `nl` layers, wait for the last of them
+            off.set_idx_on_gpu(idx, 0)
+            for l2 in range(2, nl + 2):
+                off._wait_part(l2)
+            return None
 
     row = HKV * D * es
     algo = {
@@ -99,6 +123,9 @@ def main():
         "sparse_packed": 2.0 * (k_sel + tail) * row,
         "gather": 2.0 * k_sel * row + 4.0 * k_sel,
         "copy": 2.0 * (n + tail) * row,
+        "h2d": 2.0 * k_sel * row,
+        "offload_memcpy": 2.0 * k_sel * row * nl,
+        "offload_zero_copy": 2.0 * k_sel * row * nl,
     }[args.op]
     stream = torch.cuda.current_stream()
     for i in range(args.warmup):
