@@ -124,6 +124,9 @@ class OmniKVMultiStageCache:
         self._copy_stream: Optional[torch.cuda.Stream] = None
         self._worker: Optional[threading.Thread] = None
         self._prefill_len: Optional[int] = None
+        # static decode (enable_static_decode): lengths and write positions live on the device
+        self._static = False
+        self._pos = self._len32 = self._tail_pos = self._tail_len32 = None
 
     # ------------------------------------------------------------ storage
     def _gpu_store(self, layer_idx, like: torch.Tensor, n_first: int) -> _Store:
@@ -150,12 +153,55 @@ class OmniKVMultiStageCache:
         return self._seen_tokens
 
     # ------------------------------------------------------------ reference API
+    # ------------------------------------------------------------ static decode (graph capture)
+    def enable_static_decode(self) -> None:
+        """After the prefill: switch the decode path to one whose launches never change
+        shape, so that a whole decode step can be captured in a HIP graph and replayed.
+        Sequence lengths and append positions become device scalars (the kernels read
+        per-request lengths from device memory); every buffer a step touches is
+        preallocated.  Not available with real_offload (its staging needs the host)."""
+        if self.real_offload:
+            raise NotImplementedError("static decode keeps every layer on the GPU (real_offload=False)")
+        if self._static:
+            return
+        any_store = next(iter(self._store.values()))
+        dev = any_store.k.device
+        n = self._seen_tokens
+        for layer_idx, sparse in ((i, s[0]) for i, s in self.layer_state.items()):
+            st = self._store[layer_idx]
+            if sparse:
+                if layer_idx not in self._tail:
+                    b, hkv, _, d = st.k.shape
+                    self._tail[layer_idx] = _Store(b, self.max_new_tokens, hkv, d, st.k.dtype, dev)
+            else:
+                st.reserve(n + self.max_new_tokens)
+        tails = [t.len for t in self._tail.values()]
+        t0 = tails[0] if tails else 0
+        self._pos = torch.tensor([n], dtype=torch.int64, device=dev)
+        self._len32 = torch.tensor([n + 1], dtype=torch.int32, device=dev)
+        self._tail_pos = torch.tensor([t0], dtype=torch.int64, device=dev)
+        self._tail_len32 = torch.tensor([t0 + 1], dtype=torch.int32, device=dev)
+        self._static = True
+
+    def advance_static(self) -> None:
+        """End of a static decode step: one more token everywhere (device-side adds)."""
+        self._pos += 1
+        self._len32 += 1
+        self._tail_pos += 1
+        self._tail_len32 += 1
+
     def append(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int) -> None:
         """Store the new rows of `layer_idx` (what update() does before it returns;
         modeling/spec_cache.py:308-369)."""
         if layer_idx == 0:
             self._seen_tokens += key_states.shape[-2]
         sparse = self.layer_state[layer_idx][0]
+        if self._static:
+            st = self._tail[layer_idx] if sparse else self._store[layer_idx]
+            where = self._tail_pos if sparse else self._pos
+            st.k.index_copy_(2, where, key_states)
+            st.v.index_copy_(2, where, value_states)
+            return
         if sparse and self.stage != "prefill":
             tl = self._tail.get(layer_idx)
             if tl is None:
@@ -320,6 +366,15 @@ class OmniKVMultiStageCache:
     def attend(self, query_states: torch.Tensor, layer_idx: int, scale: Optional[float] = None) -> torch.Tensor:
         """Decode attention of `layer_idx` over what update() would have returned,
         without building it.  query_states: (bsz, Hq, 1, D); returns (bsz, Hq, D)."""
+        if self._static:
+            st = self._store[layer_idx]
+            if self.layer_state[layer_idx][0]:
+                tl = self._tail[layer_idx]
+                kview, vview = st.views()
+                return ops.sparse_attn(query_states, kview, vview, idx=self._idx[self.layer_state[layer_idx][1]],
+                                       tail_k=tl.k, tail_v=tl.v, tail_len=tl.capacity, tail_lens=self._tail_len32,
+                                       scale=scale)
+            return ops.dense_attn(query_states, st.k, st.v, seq_len=st.capacity, seq_lens=self._len32, scale=scale)
         if self.layer_state[layer_idx][0] and self.stage != "prefill":
             sel = self.layer_state[layer_idx][1]
             tk = self.tail_k.get(layer_idx)
@@ -339,6 +394,17 @@ class OmniKVMultiStageCache:
         """Filter layer: dense attention and the filter-layer scores in one pass over
         K, then top-k and set_idx_on_gpu (modeling/omnikv.py:189-212 followed by the
         layer's own attention).  Returns (attention output, idx int32 (bsz, k))."""
+        if self._static:
+            st = self._store[layer_idx]
+            out, scores = ops.dense_attn(query_states, st.k, st.v, seq_len=st.capacity, seq_lens=self._len32,
+                                         selector=selector_cls, score_len=consider_len, scale=scale)
+            k = min(num_selected_tokens, consider_len)
+            buf = self._idx.get(layer_idx)
+            if buf is None or buf.shape[1] != k:
+                buf = torch.empty((scores.shape[0], k), dtype=torch.int32, device=scores.device)
+                self._idx[layer_idx] = buf  # the sparse layers keep reading this very buffer
+            ops.topk(scores, k, out=buf)
+            return out, buf
         kview, vview = self._store[layer_idx].views()
         out, scores = ops.dense_attn(query_states, kview, vview, selector=selector_cls, score_len=consider_len,
                                      scale=scale)

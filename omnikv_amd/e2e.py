@@ -31,6 +31,7 @@ def main():
     ap.add_argument("--real-offload", action="store_true")
     ap.add_argument("--offload-mode", default="zero_copy", choices=["zero_copy", "memcpy"])
     ap.add_argument("--full-attention", action="store_true", help="no selection: every layer attends to everything")
+    ap.add_argument("--graph", action="store_true", help="replay the decode step from a HIP graph")
     args = ap.parse_args()
 
     dev = torch.device("cuda:0")
@@ -50,29 +51,39 @@ def main():
 
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    logits, cache = lm.forward(ids, None, max_new_tokens=args.steps + 8, offload_mode=args.offload_mode)
+    logits, cache = lm.forward(ids, None, max_new_tokens=args.steps + 16, offload_mode=args.offload_mode)
     torch.cuda.synchronize()
     prefill_s = time.perf_counter() - t0
     tok = logits[:, -1].argmax(-1, keepdim=True)
     toks = [int(tok)]
-    for _ in range(3):  # warm-up steps (workspace growth, first selection)
-        logits, cache = lm.forward(tok, cache)
-        tok = logits[:, -1].argmax(-1, keepdim=True)
-        toks.append(int(tok))
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        logits, cache = lm.forward(tok, cache)
-        tok = logits[:, -1].argmax(-1, keepdim=True)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
+    if args.graph:
+        graph, token, _ = lm.capture_decode(cache, tok, warmup=3)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        toks.append(int(token))
+    else:
+        for _ in range(3):  # warm-up steps (workspace growth, first selection)
+            logits, cache = lm.forward(tok, cache)
+            tok = logits[:, -1].argmax(-1, keepdim=True)
+            toks.append(int(tok))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            logits, cache = lm.forward(tok, cache)
+            tok = logits[:, -1].argmax(-1, keepdim=True)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
     if args.real_offload:
         cache._join_worker()
     print(json.dumps({
         "model": f"random-init Llama-3-8B shape, {args.layers} layers, bf16", "context": args.ctx,
         "decode_steps": args.steps, "select_layers": sel, "selected": int(args.ratio * args.ctx),
         "selector": args.selector, "real_offload": bool(args.real_offload and not args.full_attention),
-        "offload_mode": args.offload_mode if args.real_offload else None, "full_attention": args.full_attention,
+        "offload_mode": args.offload_mode if args.real_offload else None, "full_attention": args.full_attention, "launch": "hip_graph_replay" if args.graph else "eager",
         "prefill_s": prefill_s, "decode_ms_per_token": dt * 1e3 / args.steps, "decode_tokens_per_s": args.steps / dt,
         "hbm_gb_allocated": round(torch.cuda.max_memory_allocated() / 1e9, 1),
         "first_tokens": toks,

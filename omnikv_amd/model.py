@@ -222,12 +222,41 @@ class OmniKVMulLM(nn.Module):
         if not isinstance(past_key_values, self.cache_cls):
             past_key_values = self.new_cache(**cache_kwargs)
         past_key_values.stage = "decoding" if n == 1 else "prefill"
-        if position_ids is None:
+        static = n == 1 and getattr(past_key_values, "_static", False)
+        if static:
+            position_ids = past_key_values._pos.view(1, 1).expand(input_ids.shape[0], -1)
+        elif position_ids is None:
             start = past_key_values.get_seq_length()
             position_ids = torch.arange(start, start + n, device=input_ids.device)[None].expand(input_ids.shape[0], -1)
         h = self.model(input_ids, position_ids, past_key_values)
         logits = self.lm_head(h[:, -1:]).float()
+        if static:
+            past_key_values.advance_static()
         return logits, past_key_values
+
+    @torch.no_grad()
+    def capture_decode(self, cache: OmniKVMultiStageCache, first_token: torch.Tensor, warmup: int = 2):
+        """Capture one greedy decode step in a HIP graph.  Returns (graph, token, logits):
+        each graph.replay() consumes `token` (1, 1), writes the step's fp32 logits into
+        `logits` and the argmax back into `token`, and moves every length on the device
+        by one -- a generation loop with no host work per token besides the replay."""
+        if "last" not in self.config.get("selector_cls", "softmax_before_last"):
+            raise NotImplementedError("the window selectors keep a host-side window; capture the `last` family")
+        cache.enable_static_decode()
+        token = first_token.clone().view(1, 1)
+        stream = torch.cuda.Stream(device=token.device)
+        stream.wait_stream(torch.cuda.current_stream(token.device))
+        with torch.cuda.stream(stream):
+            for _ in range(warmup):  # eager steps on the capture stream: workspaces, first selection
+                logits, _ = self.forward(token, cache)
+                token.copy_(logits[:, -1].argmax(-1, keepdim=True))
+            stream.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                logits, _ = self.forward(token, cache)
+                token.copy_(logits[:, -1].argmax(-1, keepdim=True))
+        torch.cuda.current_stream(token.device).wait_stream(stream)
+        return graph, token, logits
 
     @torch.no_grad()
     def generate_greedy(self, input_ids, num_tokens: int, **cache_kwargs) -> Tuple[torch.Tensor, List[torch.Tensor]]:

@@ -138,3 +138,36 @@ def test_generate_greedy_and_error_paths():
     _, cache = lm2.forward(ids, None)
     with pytest.raises(ValueError):  # modeling/omnikv.py:213-214
         lm2.forward(ids[:, :1], cache)
+
+
+@pytest.mark.parametrize("selector_cls", ["last", "softmax_before_last"])
+def test_graph_replayed_decode_matches_eager(selector_cls):
+    """A decode step captured in a HIP graph (device-side lengths and positions) must
+    reproduce the eager path token for token and logit for logit on every replay."""
+    cfg = _config(selector_cls, False)
+    ids = torch.randint(0, SHAPE.vocab_size, (1, 400), generator=torch.Generator().manual_seed(4)).to(DEV)
+    steps = 7
+
+    def fresh():
+        lm = OmniKVMulLM(SHAPE, _config(selector_cls, False)).float().to(DEV)
+        lm.init_weights(seed=11, std=0.08)
+        return lm
+
+    lm = fresh()
+    eager_toks, eager_logits = lm.generate_greedy(ids, steps + 4, max_new_tokens=32)
+    lm2 = fresh()
+    logits, cache = lm2.forward(ids, None, max_new_tokens=32)
+    assert torch.equal(logits, eager_logits[0])
+    tok = logits[:, -1].argmax(-1, keepdim=True)
+    graph, token, glogits = lm2.capture_decode(cache, tok, warmup=2)  # two eager static steps, then capture
+    assert int(token) == int(eager_toks[0, 2])
+    for t in range(steps):
+        graph.replay()
+        torch.cuda.synchronize()
+        # other work between replays, as a real loop would have
+        _ = (glogits.clone() * 2).sum().item()
+        assert (glogits - eager_logits[3 + t]).abs().max() < 1e-4, t
+        assert int(token) == int(eager_toks[0, 3 + t]), t
+    assert int(cache._len32) == 400 + 1 + 2 + steps  # capture itself executes nothing
+    with pytest.raises(NotImplementedError):
+        OmniKVMulLM(SHAPE, _config("uniform", False)).to(DEV).capture_decode(cache, tok)
