@@ -63,7 +63,8 @@ enum okv_op {
   OKV_OP_SCORE = 0,
   OKV_OP_TOPK = 1,
   OKV_OP_DENSE_ATTN = 2, /* with or without the fused score output */
-  OKV_OP_SPARSE_ATTN = 3
+  OKV_OP_SPARSE_ATTN = 3,
+  OKV_OP_SCORE_WINDOW = 4
 };
 
 typedef struct okv_kv_layout {
@@ -125,6 +126,27 @@ int okv_score(const void* q, const void* k_base, const okv_kv_layout_t* layout,
               const int32_t* score_lens, int32_t max_score_len, int32_t batch,
               int32_t head_reduce, int32_t normalise, float scale, float* scores,
               int64_t score_stride, void* ws, size_t ws_bytes, okv_stream_t stream);
+
+/*
+ * Window selectors.  q holds the last `window` query positions of every q head
+ * (element (b, h, w, d) at q + b*q_batch_stride + h*q_head_stride + w*q_pos_stride + d,
+ * strides in elements, multiples of 8; position 0 is the oldest).  For each request b
+ * and token t < score_len:
+ *   m[w][t]   = max_h softmax over t of (scale * <q[b][h][w], K[b][t][h / group]>)
+ *   uniform (exp_decay = 0):  scores[b][t] = ((m[0] + m[1]) + m[2]) + ...
+ *   exp     (exp_decay = 1):  scores[b][t] = ((m[0]/2 + m[1])/2 + m[2]) ...
+ * i.e. the additions in the order of the loops they replace:
+ * select_tokens_by_attn_universal, branches `uniform` and `exp`,
+ * modeling/omnikv.py:59-103.  K is read twice in total, not `window` times.
+ * 16-bit contiguous K, at most 8 kv heads, window * group <= 64; anything else
+ * returns OKV_ERR_UNSUPPORTED (callers then score position by position with
+ * okv_score).  Workspace: okv_workspace_bytes(OKV_OP_SCORE_WINDOW, ...).
+ */
+int okv_score_window(const void* q, int64_t q_batch_stride, int64_t q_head_stride,
+                     int64_t q_pos_stride, int32_t window, int32_t exp_decay, const void* k_base,
+                     const okv_kv_layout_t* layout, const int32_t* score_lens,
+                     int32_t max_score_len, int32_t batch, float scale, float* scores,
+                     int64_t score_stride, void* ws, size_t ws_bytes, okv_stream_t stream);
 
 /*
  * Per-request top-k of fp32 scores.  Writes the k_b = min(k_per_seg[b], len_b)

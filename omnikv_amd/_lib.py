@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(_PKG, "libomnikv_hip.so")
 OKV_F32, OKV_BF16, OKV_F16 = 0, 1, 2
 OKV_REDUCE_MAX, OKV_REDUCE_SUM = 0, 1
 OKV_NORM_RAW, OKV_NORM_SOFTMAX = 0, 1
-OKV_OP_SCORE, OKV_OP_TOPK, OKV_OP_DENSE_ATTN, OKV_OP_SPARSE_ATTN = 0, 1, 2, 3
+OKV_OP_SCORE, OKV_OP_TOPK, OKV_OP_DENSE_ATTN, OKV_OP_SPARSE_ATTN, OKV_OP_SCORE_WINDOW = 0, 1, 2, 3, 4
 
 EXPORTS = (
     "okv_strerror",
@@ -24,6 +24,7 @@ EXPORTS = (
     "okv_workspace_bytes",
     "okv_set_option",
     "okv_score",
+    "okv_score_window",
     "okv_topk",
     "okv_dense_attn",
     "okv_sparse_attn",
@@ -81,6 +82,9 @@ def _declare(l):
     l.okv_set_option.argtypes = [C.c_char_p, C.c_int]
     l.okv_score.restype = C.c_int
     l.okv_score.argtypes = [vp, vp, C.POINTER(KVLayout), vp, i32, i32, i32, i32, f32, vp, i64, vp, sz, vp]
+    l.okv_score_window.restype = C.c_int
+    l.okv_score_window.argtypes = [vp, i64, i64, i64, i32, i32, vp, C.POINTER(KVLayout), vp, i32, i32, f32, vp, i64,
+                                   vp, sz, vp]
     l.okv_topk.restype = C.c_int
     l.okv_topk.argtypes = [vp, i64, vp, i32, vp, i32, i32, vp, i64, vp, sz, vp]
     l.okv_dense_attn.restype = C.c_int

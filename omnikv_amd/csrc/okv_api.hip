@@ -109,6 +109,7 @@ int carve_attn_workspace(void* ws, size_t ws_bytes, int batch, int hq, int hkv, 
 }
 
 size_t topk_mb_workspace_bytes(int batch, int max_seq_len);
+size_t window_workspace_bytes(int batch, int hkv, int max_len);
 
 int validate_layout(const okv_kv_layout_t* layout, const void* k_base, const void* v_base) {
   OKV_REQUIRE(layout != nullptr, OKV_ERR_INVALID, "layout is NULL");
@@ -179,6 +180,9 @@ int okv_workspace_bytes(int op, const okv_shape_t* s, size_t* out_bytes) {
       return OKV_OK;
     case OKV_OP_TOPK:
       *out_bytes = okv::topk_mb_workspace_bytes(s->batch, s->max_seq_len);
+      return OKV_OK;
+    case OKV_OP_SCORE_WINDOW:
+      *out_bytes = okv::window_workspace_bytes(s->batch, s->num_kv_heads, s->max_seq_len);
       return OKV_OK;
     default:
       okv::set_error("unknown op %d", op);

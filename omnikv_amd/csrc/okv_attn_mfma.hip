@@ -21,21 +21,6 @@
 
 namespace okv {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
-typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
-typedef __attribute__((ext_vector_type(2))) float f32x2_t;
-typedef __attribute__((ext_vector_type(4))) float f32x4_t;
-
-__device__ __forceinline__ f32x4_t mfma16(const BF16*, const uint4& a, const uint4& b, f32x4_t c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
-                                                 __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-}
-__device__ __forceinline__ f32x4_t mfma16(const F16*, const uint4& a, const uint4& b, f32x4_t c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
-                                                __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
-}
 // two fp32 -> one dword of two 16-bit elements (first argument in the low half)
 __device__ __forceinline__ uint32_t pack2(const BF16*, float a, float b) {
   f32x2_t x = {a, b};

@@ -68,4 +68,22 @@ __device__ __forceinline__ void cvt8(const F16*, const uint4& u, float* o) {
   for (int i = 0; i < 8; ++i) o[i] = (float)h[i];
 }
 
+// ---- matrix cores: D(16x16 fp32) += A(16 rows x 32) . B(32 x 16 cols) of 16-bit elements.
+// Lane l holds A row l%16 / B column l%16, elements 8(l/16) .. +8 of the k-step, and
+// D column l%16, rows 4(l/16) .. +4.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+__device__ __forceinline__ f32x4_t mfma16(const BF16*, const uint4& a, const uint4& b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                 __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4_t mfma16(const F16*, const uint4& a, const uint4& b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
+                                                __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+}
 }  // namespace okv

@@ -1,0 +1,405 @@
+// Window selectors (`uniform`, `exp`): the score of a token is a sum over the last W
+// query positions of the head-max of each position's softmax over the tokens
+// (modeling/omnikv.py:59-105).  The reference runs W separate q.K^T / softmax / max
+// passes; here the W x Hq query rows ride together through the matrix cores, so K is
+// read twice in total instead of W times:
+//
+//   pass 1  window_lse_mfma    per (position, head): log-sum-exp of its logits over the
+//                              tokens, split-context partials + a small merge
+//   pass 2  window_score_mfma  logits again, probabilities exp(logit - lse), max over the
+//                              heads (lane swaps inside a kv head, LDS atomics across kv
+//                              heads), then the sum over the positions in the
+//                              reference's order of additions
+//
+// The B operand of a kv head g holds its W*G query rows as columns: column c is
+// position c/G, q head g*G + c%G; up to four 16-column blocks (W*G <= 64).
+#include <math.h>
+
+#include "okv_device.h"
+#include "okv_internal.h"
+
+namespace okv {
+
+constexpr int kWinCols = 64;  // columns (positions x q heads of one kv head) per kv head
+
+struct WindowArgs {
+  const void* q;
+  int64_t q_batch_stride, q_head_stride, q_pos_stride;  // elements
+  const void* k_base;
+  int64_t token_stride, head_stride, batch_stride;
+  const int32_t* score_lens;
+  int32_t max_score_len;
+  int32_t window, group, hkv;
+  float scale;
+  int32_t split_rows, max_splits;
+  float* part;  // [batch][hkv][kWinCols][max_splits]  log2-domain partial lse
+  float* lse;   // [batch][hkv][kWinCols]              log2-domain lse
+};
+
+__device__ __forceinline__ int win_len(const WindowArgs& a, int b) {
+  return a.score_lens ? min(a.score_lens[b], a.max_score_len) : a.max_score_len;
+}
+
+// q fragments of kv head g: qf[cb][s] = elements 32s + 8(l/16) .. +8 of column 16cb + l%16
+template <typename T, int NCB>
+__device__ __forceinline__ void load_window_q(const WindowArgs& a, int b, int g, int r16, int j4,
+                                              uint4 (&qf)[NCB][4]) {
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) {
+    const int c = 16 * cb + r16;
+    const int w = c / a.group, hg = c % a.group;
+    const bool valid = w < a.window;
+    const T* qp = reinterpret_cast<const T*>(a.q) + (int64_t)b * a.q_batch_stride +
+                  (int64_t)(g * a.group + hg) * a.q_head_stride +
+                  (int64_t)(valid ? w : 0) * a.q_pos_stride + 8 * j4;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const uint4 v = *reinterpret_cast<const uint4*>(qp + 32 * s);
+      qf[cb][s] = valid ? v : make_uint4(0, 0, 0, 0);
+    }
+  }
+}
+
+// ------------------------------------------------------------------ pass 1
+// grid (kv heads, splits, batch), 256 threads; wave w of the block takes the 16-row
+// tiles begin + 16(w + 4n) of its split.
+template <typename T, int NCB>
+__global__ __launch_bounds__(256) void window_lse_mfma(WindowArgs a) {
+  __shared__ float sm[16][16 * NCB], sl[16][16 * NCB];
+  const int g = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
+  const int A = win_len(a, b);
+  const int begin = split * a.split_rows;
+  const int end = min(begin + a.split_rows, A);
+  if (begin >= end) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r16 = lane & 15, j4 = lane >> 4;
+
+  uint4 qf[NCB][4];
+  load_window_q<T, NCB>(a, b, g, r16, j4, qf);
+  const T* kb = reinterpret_cast<const T*>(a.k_base) + (int64_t)b * a.batch_stride +
+                (int64_t)g * a.head_stride + 8 * j4;
+  const uint32_t ts = (uint32_t)a.token_stride;
+  const int last = end - 1;
+  auto load_tile = [&](int tbase, uint4 (&kf)[4]) {
+    int r = tbase + r16;
+    r = r < last ? r : last;
+    const T* kp = kb + (uint64_t)(uint32_t)r * ts;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) kf[s] = *reinterpret_cast<const uint4*>(kp + 32 * s);
+  };
+  const float sl2 = a.scale * kLog2e;
+  float m[NCB], l[NCB];  // per column block: state of (column r16, lane row j4), m in raw units
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) {
+    m[cb] = -INFINITY;
+    l[cb] = 0.f;
+  }
+  auto compute = [&](int tbase, const uint4 (&kf)[4]) {
+    const int row0 = tbase + 4 * j4;
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) {
+      f32x4_t S = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 4; ++s) S = mfma16((const T*)nullptr, kf[s], qf[cb][s], S);
+      float sv[4] = {S[0], S[1], S[2], S[3]};
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (row0 + i >= end) sv[i] = -INFINITY;
+      const float mn = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), m[cb]);
+      const float ms = mn == -INFINITY ? 0.f : mn;
+      const float alpha = __builtin_amdgcn_exp2f((m[cb] - ms) * sl2);
+      float p = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) p += __builtin_amdgcn_exp2f((sv[i] - ms) * sl2);
+      l[cb] = fmaf(l[cb], alpha, p);
+      m[cb] = mn;
+    }
+  };
+  {
+    uint4 kA[4], kB[4];
+    int t = begin + wave * 16;
+    if (t < end) {
+      const int t_last = t + ((last - t) >> 6 << 6);
+      load_tile(t, kA);
+      if (t == t_last) {
+        compute(t, kA);
+      } else {
+        while (true) {  // every load unconditional (clamped): the next tile stays in flight
+          load_tile(min(t + 64, t_last), kB);
+          compute(t, kA);
+          t += 64;
+          load_tile(min(t + 64, t_last), kA);
+          compute(t, kB);
+          if (t == t_last) break;
+          t += 64;
+          if (t == t_last) {
+            compute(t, kA);
+            break;
+          }
+        }
+      }
+    }
+  }
+  const int grp = wave * 4 + j4;
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) {
+    sm[grp][16 * cb + r16] = m[cb];
+    sl[grp][16 * cb + r16] = l[cb];
+  }
+  __syncthreads();
+  if (threadIdx.x < 16 * NCB) {
+    const int c = threadIdx.x;
+    float M = -INFINITY;
+#pragma unroll
+    for (int x = 0; x < 16; ++x) M = fmaxf(M, sm[x][c]);
+    float den = 0.f;
+#pragma unroll
+    for (int x = 0; x < 16; ++x) {
+      const float mm = sm[x][c];
+      den = fmaf(sl[x][c], mm == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((mm - M) * sl2), den);
+    }
+    a.part[((int64_t)(b * a.hkv + g) * kWinCols + c) * a.max_splits + split] =
+        M == -INFINITY ? -INFINITY : M * sl2 + log2f(den);
+  }
+}
+
+// grid (batch * kv heads), 256 threads: 64 columns x 4 split lanes, independent loads
+__global__ __launch_bounds__(256) void window_lse_merge(WindowArgs a) {
+  __shared__ float sM[4][kWinCols], sD[4][kWinCols];
+  const int bg = blockIdx.x, b = bg / a.hkv, c = threadIdx.x & 63, sl = threadIdx.x >> 6;
+  const int A = win_len(a, b);
+  const int ns = (A + a.split_rows - 1) / a.split_rows;
+  const float* p = a.part + ((int64_t)bg * kWinCols + c) * a.max_splits;
+  float M = -INFINITY, den = 0.f;
+  constexpr int U = 8;
+  for (int s0 = sl; s0 < ns; s0 += 4 * U) {
+    float x[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) x[u] = s0 + 4 * u < ns ? p[s0 + 4 * u] : -INFINITY;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const float mn = fmaxf(M, x[u]);
+      if (mn != -INFINITY) {
+        den = fmaf(den, exp2f(M - mn), exp2f(x[u] - mn));
+        M = mn;
+      }
+    }
+  }
+  sM[sl][c] = M;
+  sD[sl][c] = den;
+  __syncthreads();
+  if (sl == 0) {
+    float Mt = fmaxf(fmaxf(sM[0][c], sM[1][c]), fmaxf(sM[2][c], sM[3][c]));
+    float d = 0.f;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) d += sM[x][c] == -INFINITY ? 0.f : sD[x][c] * exp2f(sM[x][c] - Mt);
+    a.lse[(int64_t)bg * kWinCols + c] = Mt + log2f(d);
+  }
+}
+
+// lane i of every quad reads lane perm[i]: 0xB1 = {1,0,3,2} (xor 1), 0x4E = {2,3,0,1} (xor 2)
+template <int QUAD_PERM>
+__device__ __forceinline__ float quad_swap(float x) {
+  return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), QUAD_PERM, 0xf, 0xf, true));
+}
+
+// ------------------------------------------------------------------ pass 2
+// grid (row blocks, batch), one wave per kv head; LDS: [window][rows_per_block] bit
+// patterns of non-negative floats (their unsigned order is their numeric order).
+template <typename T, int NCB>
+__global__ __launch_bounds__(512) void window_score_mfma(WindowArgs a, int rows_per_block, int exp_decay,
+                                                         float* __restrict__ scores,
+                                                         int64_t score_stride) {
+  extern __shared__ uint32_t wmax[];
+  const int b = blockIdx.y;
+  const int A = win_len(a, b);
+  const int begin = blockIdx.x * rows_per_block;
+  const int end = min(begin + rows_per_block, A);
+  if (begin >= end) return;
+  const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int r16 = lane & 15, j4 = lane >> 4;
+
+  for (int i = threadIdx.x; i < a.window * rows_per_block; i += blockDim.x) wmax[i] = 0u;
+
+  uint4 qf[NCB][4];
+  load_window_q<T, NCB>(a, b, g, r16, j4, qf);
+  float lse[NCB];
+  int wcol[NCB];  // position of this lane's column, or -1 when the lane does not report it
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) {
+    const int c = 16 * cb + r16;
+    lse[cb] = a.lse[(int64_t)(b * a.hkv + g) * kWinCols + c];
+    wcol[cb] = (c % a.group == 0 && c / a.group < a.window) ? c / a.group : -1;
+  }
+  const T* kb = reinterpret_cast<const T*>(a.k_base) + (int64_t)b * a.batch_stride +
+                (int64_t)g * a.head_stride + 8 * j4;
+  const uint32_t ts = (uint32_t)a.token_stride;
+  const int last = end - 1;
+  auto load_tile = [&](int tbase, uint4 (&kf)[4]) {
+    int r = tbase + r16;
+    r = r < last ? r : last;
+    const T* kp = kb + (uint64_t)(uint32_t)r * ts;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) kf[s] = *reinterpret_cast<const uint4*>(kp + 32 * s);
+  };
+  const float sl2 = a.scale * kLog2e;
+  auto compute = [&](int tbase, const uint4 (&kf)[4]) {
+    const int row0 = tbase + 4 * j4 - begin;
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) {
+      f32x4_t S = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 4; ++s) S = mfma16((const T*)nullptr, kf[s], qf[cb][s], S);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float p = __builtin_amdgcn_exp2f(fmaf(S[i], sl2, -lse[cb]));
+        // max over the q heads of the kv head: neighbours inside a quad by DPP, beyond by a swap
+        if (a.group >= 2) p = fmaxf(p, quad_swap<0xB1>(p));
+        if (a.group >= 4) p = fmaxf(p, quad_swap<0x4E>(p));
+        if (a.group >= 8) p = fmaxf(p, __shfl_xor(p, 4));
+        if (wcol[cb] >= 0 && row0 + i < end - begin)
+          atomicMax(&wmax[wcol[cb] * rows_per_block + row0 + i], __float_as_uint(p));
+      }
+    }
+  };
+  __syncthreads();  // the zero fill is complete
+  {
+    // four tiles in flight per wave (one workgroup per CU has to cover the memory latency
+    // by itself); every load is unconditional, past the end it repeats the last tile
+    uint4 kf[4][4];
+    const int t_last = begin + ((last - begin) >> 4 << 4);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) load_tile(min(begin + 16 * u, t_last), kf[u]);
+    for (int t = begin; t <= t_last; t += 64) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int tt = t + 16 * u;
+        if (tt <= t_last) compute(tt, kf[u]);
+        load_tile(min(tt + 64, t_last), kf[u]);
+      }
+    }
+  }
+  __syncthreads();
+  for (int r = threadIdx.x; r < end - begin; r += blockDim.x) {
+    // the reference's order: positions oldest first, running sum (uniform) or
+    // running sum halved before each addition (exp)
+    float acc = __uint_as_float(wmax[r]);
+    for (int w = 1; w < a.window; ++w) {
+      const float v = __uint_as_float(wmax[w * rows_per_block + r]);
+      acc = exp_decay ? acc * 0.5f + v : acc + v;
+    }
+    scores[(int64_t)b * score_stride + begin + r] = acc;
+  }
+}
+
+// ------------------------------------------------------------------ host
+static int window_split_rows(int batch, int hkv, int max_len, int cus) {
+  const int64_t capacity = (int64_t)cus * 3;
+  const int64_t work = (int64_t)max_len * hkv * batch;
+  int64_t rows = (work + capacity - 1) / capacity;
+  rows = (rows + 63) / 64 * 64;
+  return (int)(rows < 64 ? 64 : rows);
+}
+
+static int num_cus() {
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) == hipSuccess &&
+      hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+    return n;
+  return 256;
+}
+
+size_t window_workspace_bytes(int batch, int hkv, int max_len) {
+  const int sr = window_split_rows(batch, hkv, max_len, num_cus());
+  const int splits = (max_len + sr - 1) / sr;
+  return (size_t)batch * hkv * kWinCols * ((size_t)(splits > 0 ? splits : 1) + 1) * sizeof(float) + 512;
+}
+
+template <typename T, int NCB>
+static void launch_window(WindowArgs a, int batch, int exp_decay, float* scores, int64_t score_stride,
+                          int cus, hipStream_t stream) {
+  hipLaunchKernelGGL((window_lse_mfma<T, NCB>), dim3(a.hkv, a.max_splits, batch), dim3(256), 0, stream, a);
+  hipLaunchKernelGGL(window_lse_merge, dim3(batch * a.hkv), dim3(256), 0, stream, a);
+  // one round of row blocks, one block of `hkv` waves per CU; LDS bounds the rows
+  int64_t per = ((int64_t)a.max_score_len * batch + cus - 1) / cus;
+  int rpb = (int)((per + 15) / 16 * 16);
+  if (rpb < 64) rpb = 64;
+  const int cap = (48 * 1024 / 4 / a.window) / 16 * 16;
+  if (rpb > cap) rpb = cap;
+  dim3 grid((a.max_score_len + rpb - 1) / rpb, batch);
+  hipLaunchKernelGGL((window_score_mfma<T, NCB>), grid, dim3(64 * a.hkv),
+                     (size_t)a.window * rpb * sizeof(uint32_t), stream, a, rpb, exp_decay, scores,
+                     score_stride);
+}
+
+template <typename T>
+static void launch_window_t(const WindowArgs& a, int batch, int exp_decay, float* scores,
+                            int64_t score_stride, int cus, hipStream_t stream) {
+  const int ncb = (a.window * a.group + 15) / 16;
+  switch (ncb) {
+    case 1: launch_window<T, 1>(a, batch, exp_decay, scores, score_stride, cus, stream); break;
+    case 2: launch_window<T, 2>(a, batch, exp_decay, scores, score_stride, cus, stream); break;
+    case 3: launch_window<T, 3>(a, batch, exp_decay, scores, score_stride, cus, stream); break;
+    default: launch_window<T, 4>(a, batch, exp_decay, scores, score_stride, cus, stream); break;
+  }
+}
+
+}  // namespace okv
+
+using namespace okv;
+
+extern "C" int okv_score_window(const void* q, int64_t q_batch_stride, int64_t q_head_stride,
+                                int64_t q_pos_stride, int32_t window, int32_t exp_decay,
+                                const void* k_base, const okv_kv_layout_t* layout,
+                                const int32_t* score_lens, int32_t max_score_len, int32_t batch,
+                                float scale, float* scores, int64_t score_stride, void* ws,
+                                size_t ws_bytes, okv_stream_t stream) {
+  int rc = validate_layout(layout, k_base, k_base);
+  if (rc) return rc;
+  OKV_REQUIRE(q && scores, OKV_ERR_INVALID, "q or scores is NULL");
+  OKV_REQUIRE(batch >= 1 && max_score_len >= 0 && window >= 1, OKV_ERR_INVALID,
+              "bad batch, length or window");
+  OKV_REQUIRE(score_stride >= max_score_len, OKV_ERR_INVALID, "score_stride < max_score_len");
+  OKV_REQUIRE(((uintptr_t)q & 15) == 0 && q_batch_stride % 8 == 0 && q_head_stride % 8 == 0 &&
+                  q_pos_stride % 8 == 0,
+              OKV_ERR_INVALID, "q must be 16-byte aligned with strides that are multiples of 8");
+  const int hkv = layout->num_kv_heads, group = layout->num_q_heads / hkv;
+  OKV_REQUIRE(layout->dtype == OKV_BF16 || layout->dtype == OKV_F16, OKV_ERR_UNSUPPORTED,
+              "window scoring runs on the matrix cores: 16-bit K only");
+  OKV_REQUIRE(layout->page_table == nullptr, OKV_ERR_UNSUPPORTED, "window scoring reads contiguous K only");
+  OKV_REQUIRE(window * group <= kWinCols, OKV_ERR_UNSUPPORTED,
+              "window %d x group %d exceeds %d query rows per kv head", window, group, kWinCols);
+  OKV_REQUIRE(hkv <= 8, OKV_ERR_UNSUPPORTED, "more than 8 kv heads");
+  OKV_REQUIRE(layout->token_stride < (1ll << 31), OKV_ERR_UNSUPPORTED, "token stride too large");
+  if (max_score_len == 0) return OKV_OK;
+  OKV_REQUIRE(ws != nullptr && ws_bytes >= window_workspace_bytes(batch, hkv, max_score_len),
+              OKV_ERR_WORKSPACE, "workspace too small: have %zu, need %zu", ws_bytes,
+              window_workspace_bytes(batch, hkv, max_score_len));
+  const int cus = num_cus();
+  WindowArgs a;
+  a.q = q;
+  a.q_batch_stride = q_batch_stride;
+  a.q_head_stride = q_head_stride;
+  a.q_pos_stride = q_pos_stride;
+  a.k_base = k_base;
+  a.token_stride = layout->token_stride;
+  a.head_stride = layout->head_stride;
+  a.batch_stride = layout->batch_stride;
+  a.score_lens = score_lens;
+  a.max_score_len = max_score_len;
+  a.window = window;
+  a.group = group;
+  a.hkv = hkv;
+  a.scale = scale;
+  a.split_rows = window_split_rows(batch, hkv, max_score_len, cus);
+  a.max_splits = (max_score_len + a.split_rows - 1) / a.split_rows;
+  char* p = (char*)(((uintptr_t)ws + 255) & ~(uintptr_t)255);
+  a.part = (float*)p;
+  a.lse = a.part + (size_t)batch * hkv * kWinCols * a.max_splits;
+  if (layout->dtype == OKV_BF16)
+    launch_window_t<BF16>(a, batch, exp_decay != 0, scores, score_stride, cus, (hipStream_t)stream);
+  else
+    launch_window_t<F16>(a, batch, exp_decay != 0, scores, score_stride, cus, (hipStream_t)stream);
+  OKV_HIP_CHECK(hipGetLastError());
+  return OKV_OK;
+}

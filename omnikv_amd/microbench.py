@@ -25,7 +25,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--op", required=True,
                     choices=["dense", "fused", "score", "topk", "sparse", "sparse_packed", "gather", "copy",
-                             "offload_memcpy", "offload_zero_copy", "h2d"])
+                             "offload_memcpy", "offload_zero_copy", "h2d", "window", "window_loop"])
+    ap.add_argument("--window", type=int, default=16, help="query positions of the window selectors")
     ap.add_argument("--cpu-threads", type=int, default=8, help="packing threads of the offload tier")
     ap.add_argument("--ctx", type=int, default=131072)
     ap.add_argument("--ratio", type=float, default=0.067)
@@ -69,6 +70,8 @@ def main():
     packed = [(ops.gather_rows(ks[l][:, :, :n], idx), ops.gather_rows(vs[l][:, :, :n], idx)) for l in range(nl)] \
         if args.op == "sparse_packed" else None
     dst = torch.empty_like(ks[0]) if args.op == "copy" else None
+    qw = [torch.randn((1, HQ, args.window, D), generator=gen, device=dev).to(dtype) for _ in range(nl)] \
+        if args.op.startswith("window") else None
     off = None
     if args.op.startswith("offload") or args.op == "h2d":
         # one offloaded layer group: `nl` layers whose prompt K/V live in pinned host memory
@@ -94,6 +97,14 @@ def main():
             return ops.score(qs[l], ks[l][:, :, :n], selector=args.selector)
         if args.op == "topk":
             return ops.topk(scores, k_sel)
+        if args.op == "window":
+            return ops.score_window(qw[l], ks[l][:, :, :n], selector="uniform")
+        if args.op == "window_loop":
+            acc = None
+            for t in range(args.window):
+                s = ops.score(qw[l][:, :, t:t + 1], ks[l][:, :, :n], selector="softmax_before_last")
+                acc = s if acc is None else acc + s
+            return acc
         if args.op == "sparse":
             return ops.sparse_attn(qs[l], ks[l][:, :, :n], vs[l][:, :, :n], idx=idx,
                                    tail_k=ks[l][:, :, n:], tail_v=vs[l][:, :, n:])
@@ -119,6 +130,8 @@ def main():
         "fused": 2.0 * (n + tail) * row + 4.0 * n,
         "score": 1.0 * n * row + 4.0 * n,
         "topk": 4.0 * n + 4.0 * k_sel,
+        "window": 1.0 * n * row + 4.0 * n,  # one reading of K; the kernels read it twice
+        "window_loop": 1.0 * n * row + 4.0 * n,
         "sparse": 2.0 * (k_sel + tail) * row + 4.0 * k_sel,
         "sparse_packed": 2.0 * (k_sel + tail) * row,
         "gather": 2.0 * k_sel * row + 4.0 * k_sel,

@@ -140,6 +140,40 @@ def score(q, k, score_len: Optional[int] = None, selector: str = "last", scale: 
     return out
 
 
+def window_supported(q: torch.Tensor, k) -> bool:
+    """Whether score_window takes these operands (else: one `score` call per position)."""
+    if isinstance(k, PagedKV) or q.dim() != 4 or q.dtype not in (torch.bfloat16, torch.float16):
+        return False
+    hq, w = q.shape[1], q.shape[2]
+    hkv = k.shape[1]
+    return k.dtype == q.dtype and hkv <= 8 and hq % hkv == 0 and w * (hq // hkv) <= 64
+
+
+def score_window(q, k, score_len: Optional[int] = None, selector: str = "uniform", scale: Optional[float] = None,
+                 score_lens: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """(bsz, score_len) fp32 scores of the window selectors; okv_score_window.
+    q: (bsz, Hq, W, D), the last W query positions, oldest first."""
+    _require_gpu(q, "q")
+    if selector not in ("uniform", "exp"):
+        raise ValueError(f"selector {selector!r} is not a window selector")
+    if q.dim() != 4 or q.stride(3) != 1:
+        raise ValueError("q must be (bsz, Hq, W, D) with contiguous D")
+    hq, w, d = q.shape[1], q.shape[2], q.shape[3]
+    lay, kp, _, batch, n = _layout(k, None, hq)
+    if score_len is None:
+        score_len = n
+    if out is None:
+        out = torch.empty((batch, score_len), dtype=torch.float32, device=q.device)
+    nbytes = workspace_bytes(_lib.OKV_OP_SCORE_WINDOW, batch, hq, lay.num_kv_heads, d, score_len)
+    ws = _workspace(q.device, nbytes)
+    check(lib().okv_score_window(
+        q.data_ptr(), q.stride(0), q.stride(1), q.stride(2), w, int(selector == "exp"), kp, C.byref(lay),
+        _lens(score_lens, batch, "score_lens"), score_len, batch,
+        scale if scale is not None else 1.0 / math.sqrt(d),
+        out.data_ptr(), out.stride(0), ws.data_ptr(), ws.numel(), _stream_ptr(q.device)))
+    return out
+
+
 def topk(scores: torch.Tensor, k: int, seq_lens: Optional[torch.Tensor] = None,
          k_per_seg: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """(bsz, min(k, N)) int32 ascending indices of the k largest scores; okv_topk."""

@@ -37,7 +37,9 @@ def select_from_query(query_states: torch.Tensor, key_cache: torch.Tensor, num_s
         # modeling/omnikv.py:59-103: per window position softmax, head max; summed
         # (uniform) or folded with weight 1/2 per step of age (exp)
         scores = None
-        for t in range(query_states.shape[2]):
+        if ops.window_supported(query_states, key_cache):  # all positions in two passes over K
+            scores = ops.score_window(query_states, key_cache, score_len=consider_len, selector=selector_cls)
+        for t in range(query_states.shape[2] if scores is None else 0):
             s = ops.score(query_states[:, :, t: t + 1, :], key_cache, score_len=consider_len,
                           selector="softmax_before_last")
             if scores is None:

@@ -273,3 +273,76 @@ def test_topk_repeated_calls_leave_workspace_clean():
         if i % 2:
             s = torch.softmax(s * 3, dim=-1)
         _check_topk(s, max(1, int(0.067 * n)))
+
+
+# ------------------------------------------------------------------ window selectors
+def _window_inputs(n, w, hq, hkv, dtype, seed=3, bsz=1):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn((bsz, hq, w, 128), generator=g).to(dtype)
+    k = torch.randn((bsz, hkv, n, 128), generator=g)
+    k[:, :, 0] *= 4.0  # a sink token, so that the softmax is peaked like a real one
+    return q, k.to(dtype)
+
+
+@pytest.mark.parametrize("selector", ["uniform", "exp"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("w,hq,hkv,n", [(1, 32, 8, 1000), (3, 32, 8, 4096), (16, 32, 8, 4099), (16, 32, 8, 70001),
+                                        (8, 32, 4, 3000), (5, 8, 8, 2048), (7, 16, 8, 777)])
+def test_window_scores_match_oracle(selector, dtype, w, hq, hkv, n):
+    """All window positions in two passes over K (matrix cores) against the oracle's
+    position-by-position loop on the same 16-bit values."""
+    q, k = _window_inputs(n, w, hq, hkv, dtype)
+    assert ops.window_supported(q.to(DEV), k.to(DEV))
+    consider = n - 3
+    got = ops.score_window(q.to(DEV), k.to(DEV), score_len=consider, selector=selector).cpu()
+    want = orc.score_tokens(q.float(), k.float(), consider, selector)
+    assert got.shape == want.shape
+    assert _rel_err(got, want) < 1e-4
+    kk = max(1, int(0.067 * consider))
+    a = set(ops.topk(got.to(DEV), kk).cpu()[0].tolist())
+    b = set(orc.select_topk(want, kk)[0].tolist())
+    assert len(a & b) >= kk - 2
+
+
+@pytest.mark.parametrize("selector", ["uniform", "exp"])
+def test_window_scores_equal_the_per_position_kernels(selector):
+    """The fused window kernel and one okv_score call per position compute the same
+    sums in the same order: agreement to fp32 rounding of the softmax terms."""
+    q, k = _window_inputs(20000, 16, 32, 8, torch.bfloat16, seed=9)
+    qd, kd = q.to(DEV), k.to(DEV)
+    fused = ops.score_window(qd, kd, selector=selector)
+    loop = None
+    for t in range(16):
+        s = ops.score(qd[:, :, t:t + 1], kd, selector="softmax_before_last")
+        loop = s if loop is None else (loop + s if selector == "uniform" else loop * 0.5 + s)
+    assert _rel_err(fused.cpu(), loop.cpu()) < 2e-5
+    # every position's head-max softmax lies in (0, 1]: bounds of the sums
+    top = 16.0 if selector == "uniform" else 2.0
+    assert float(fused.min()) >= 0.0 and float(fused.max()) <= top
+
+
+def test_window_scores_ragged_batch_and_strided_q():
+    """Per-request lengths, and q taken as a view of a longer (bsz, Hq, L, D) tensor."""
+    lens = [5000, 37, 2048, 1]
+    q_all, k = _window_inputs(5000, 24, 32, 8, torch.bfloat16, seed=21, bsz=4)
+    q = q_all[:, :, 8:24]  # the last 16 positions: a strided view
+    sl = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    got = ops.score_window(q.to(DEV)[:, :, :], k.to(DEV), score_len=5000, selector="exp", score_lens=sl).cpu()
+    qv = q_all.to(DEV)[:, :, 8:24]
+    assert not qv.is_contiguous()
+    got_view = ops.score_window(qv, k.to(DEV), score_len=5000, selector="exp", score_lens=sl).cpu()
+    for b, n in enumerate(lens):
+        want = orc.score_tokens(q[b:b + 1].float(), k[b:b + 1].float(), n, "exp")
+        assert _rel_err(got[b:b + 1, :n], want) < 1e-4
+        assert torch.equal(got[b, :n], got_view[b, :n])
+
+
+def test_window_unsupported_shapes_are_refused():
+    q, k = _window_inputs(256, 17, 32, 8, torch.bfloat16)  # 17 positions x group 4 > 64 columns
+    assert not ops.window_supported(q.to(DEV), k.to(DEV))
+    with pytest.raises(Exception, match="unsupported"):
+        ops.score_window(q.to(DEV), k.to(DEV), selector="uniform")
+    q32, k32 = _window_inputs(256, 4, 32, 8, torch.float32)
+    assert not ops.window_supported(q32.to(DEV), k32.to(DEV))
+    with pytest.raises(Exception, match="unsupported"):
+        ops.score_window(q32.to(DEV), k32.to(DEV), selector="uniform")
