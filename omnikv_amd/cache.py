@@ -89,8 +89,13 @@ class OmniKVMultiStageCache:
     """Drop-in for the reference class of the same name (default DenseMore=True)."""
 
     def __init__(self, full_attn_layers: List, num_hidden_layers, num_wait_load_layers=2, real_offload=True,
-                 max_new_tokens: int = 1024, offload_mode: str = "zero_copy", cpu_num_threads: int = 8):
+                 max_new_tokens: int = 1024, offload_mode: str = "zero_copy", cpu_num_threads: int = 8,
+                 skip_threshold: Optional[float] = None):
         self.stage = "prefill"
+        # lazy re-selection (OmniKVLazyCache.set_out_idx, modeling/spec_cache.py:539-557): a new
+        # selection whose IoU with the one in use exceeds the threshold is dropped
+        self.skip_threshold = skip_threshold
+        self.num_skipped_selections = 0
         self.full_attn_layers = full_attn_layers
         self.num_hidden_layers = num_hidden_layers
         self.num_wait_layers = num_wait_load_layers
@@ -118,10 +123,13 @@ class OmniKVMultiStageCache:
         self._idx: Dict[int, torch.Tensor] = {}    # filter layer -> (bsz, k) int32 on the GPU
         self._part: Dict[int, torch.Tensor] = {}   # sparse layer -> (bsz, k, 2, Hkv, D) staged rows
         self._part_src: Dict[int, int] = {}        # sparse layer -> id of the idx it was gathered with
+        self._staged_for: Dict[int, int] = {}      # sparse layer -> id of the idx its rows were staged with
         self._staging: Dict[int, torch.Tensor] = {}
         self._events: Dict[int, torch.cuda.Event] = {}
         self._recorded: Dict[int, threading.Event] = {}
         self._copy_stream: Optional[torch.cuda.Stream] = None
+        self._d2h_stream: Optional[torch.cuda.Stream] = None
+        self._d2h_pending = False
         self._worker: Optional[threading.Thread] = None
         self._prefill_len: Optional[int] = None
         # static decode (enable_static_decode): lengths and write positions live on the device
@@ -223,9 +231,18 @@ class OmniKVMultiStageCache:
                 self._host_kv[layer_idx] = host
             elif host.shape[0] != n:
                 raise NotImplementedError("an offloaded layer takes its prompt in one prefill call")
-            is_last = layer_idx == self.num_hidden_layers - 1
-            host[:, 0].copy_(key_states[0].permute(1, 0, 2), non_blocking=not is_last)
-            host[:, 1].copy_(value_states[0].permute(1, 0, 2), non_blocking=not is_last)
+            # device-to-host on a stream of its own: the next layer's prefill compute runs
+            # meanwhile; the stream is drained when decoding starts (_finish_prefill_offload)
+            cur = torch.cuda.current_stream(key_states.device)
+            if self._d2h_stream is None:
+                self._d2h_stream = torch.cuda.Stream(device=key_states.device)
+            self._d2h_stream.wait_stream(cur)
+            with torch.cuda.stream(self._d2h_stream):
+                host[:, 0].copy_(key_states[0].permute(1, 0, 2), non_blocking=True)
+                host[:, 1].copy_(value_states[0].permute(1, 0, 2), non_blocking=True)
+            key_states.record_stream(self._d2h_stream)
+            value_states.record_stream(self._d2h_stream)
+            self._d2h_pending = True
             self._sync_lists(layer_idx)
             return
         st = self._gpu_store(layer_idx, key_states, key_states.shape[2])
@@ -252,6 +269,11 @@ class OmniKVMultiStageCache:
             idx = idx[None]
         idx32 = idx if idx.dtype == torch.int32 else idx.to(torch.int32)
         idx32 = idx32.contiguous()
+        old = self._idx.get(sel_layer_idx)
+        if self.skip_threshold is not None and old is not None and not self._static:
+            if get_idx_iou_score(idx32.view(-1), old.view(-1)) > self.skip_threshold:
+                self.num_skipped_selections += 1
+                return
         self._idx[sel_layer_idx] = idx32
         hi = self.layer_state[sel_layer_idx][2]
         lo = sel_layer_idx + self.num_wait_layers + 1
@@ -259,15 +281,18 @@ class OmniKVMultiStageCache:
             self.part_key.pop(i, None)
             self.part_value.pop(i, None)
             self._part_src.pop(i, None)
-        if self.real_offload and lo < hi:
+        if self.real_offload and lo < hi and self._stage_at_selection:
             self._start_offload(idx32, list(range(lo, hi)))
+
+    _stage_at_selection = True  # False: each sparse layer stages its own rows when it runs
 
     @staticmethod
     def from_dynamic_cache(cache, full_attn_layers: List, num_hidden_layers, num_wait_load_layers=2,
                            real_offload=True, **kwargs):
         """modeling/spec_cache.py:371-385; `cache` is anything with key_cache /
         value_cache lists (or transformers >= 4.54 `.layers[i].keys/.values`)."""
-        c = OmniKVMultiStageCache(full_attn_layers, num_hidden_layers, num_wait_load_layers, real_offload, **kwargs)
+        c = kwargs.pop("_cls", OmniKVMultiStageCache)(full_attn_layers, num_hidden_layers, num_wait_load_layers,
+                                                       real_offload, **kwargs)
         keys = getattr(cache, "key_cache", None)
         vals = getattr(cache, "value_cache", None)
         if keys is None and hasattr(cache, "layers"):
@@ -280,9 +305,17 @@ class OmniKVMultiStageCache:
         return c
 
     # ------------------------------------------------------------ offload tier
+    def _finish_prefill_offload(self) -> None:
+        """The prompt's host copies are complete before anything reads them (host threads
+        of the memcpy mode included)."""
+        if self._d2h_pending:
+            self._d2h_stream.synchronize()
+            self._d2h_pending = False
+
     def _start_offload(self, idx32: torch.Tensor, layers: List[int]) -> None:
         if idx32.shape[0] != 1:
             raise NotImplementedError("real_offload keeps one request")
+        self._finish_prefill_offload()
         self._join_worker()
         dev = idx32.device
         if self._copy_stream is None:
@@ -337,6 +370,10 @@ class OmniKVMultiStageCache:
 
     def _wait_part(self, layer_idx: int) -> torch.Tensor:
         """Staged rows of an offloaded layer, ordered behind their copy on the current stream."""
+        sel = self.layer_state[layer_idx][1]
+        if not self._stage_at_selection and self._staged_for.get(layer_idx) != id(self._idx[sel]):
+            self._start_offload(self._idx[sel], [layer_idx])  # this layer only, now
+            self._staged_for[layer_idx] = id(self._idx[sel])
         self._recorded[layer_idx].wait()
         torch.cuda.current_stream(self._part[layer_idx].device).wait_event(self._events[layer_idx])
         return self._part[layer_idx]
@@ -430,10 +467,36 @@ def _gather_wide(src: torch.Tensor, idx32: torch.Tensor, dst: torch.Tensor) -> N
                                 torch.cuda.current_stream(idx32.device).cuda_stream))
 
 
+class WOPackCache(OmniKVMultiStageCache):
+    """`cache_cls: without_pack` (modeling/spec_cache.py:388-520): set_idx_on_gpu only
+    records the selection; with real_offload each sparse layer fetches its own rows
+    when it runs (spec_cache.py:477-483) instead of all layers of the group being staged
+    ahead at selection time.  Without offload there is nothing to pack in this build
+    (the sparse kernel reads the rows in place), so the two classes then coincide."""
+
+    _stage_at_selection = False
+
+    @staticmethod
+    def from_dynamic_cache(cache, full_attn_layers: List, num_hidden_layers, num_wait_load_layers=2,
+                           real_offload=True, **kwargs):
+        return OmniKVMultiStageCache.from_dynamic_cache(cache, full_attn_layers, num_hidden_layers,
+                                                        num_wait_load_layers, real_offload, _cls=WOPackCache, **kwargs)
+
+
+def get_idx_iou_score(new_idx: torch.Tensor, old_idx: torch.Tensor) -> float:
+    """Overlap of two 1-D index tensors as the reference scores it
+    (modeling/spec_cache.py:10-32): |new & old| / |new| -- despite its name not divided by
+    the union.  Synchronises with the device, as the reference's Python float does."""
+    assert new_idx.dim() == 1 and old_idx.dim() == 1, "Both tensors should be 1D"
+    un = torch.cat([new_idx, old_idx], dim=0).unique().shape[0]
+    inter = new_idx.shape[0] + old_idx.shape[0] - un
+    return inter / new_idx.shape[0]
+
+
 def get_cache_cls(config):
-    """modeling/spec_cache.py:829-837, restricted to the class this build provides."""
-    name2cls = {"multi": OmniKVMultiStageCache}
+    """modeling/spec_cache.py:829-837, restricted to the classes this build provides."""
+    name2cls = {"multi": OmniKVMultiStageCache, "without_pack": WOPackCache}
     name = config.get("cache_cls", "default")
     if name not in name2cls:
-        raise NotImplementedError(f"cache_cls={name!r}: only 'multi' is built here")
+        raise NotImplementedError(f"cache_cls={name!r}: 'multi' and 'without_pack' are built here")
     return name2cls[name]

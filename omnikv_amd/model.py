@@ -212,6 +212,8 @@ class OmniKVMulLM(nn.Module):
     def new_cache(self, **kwargs) -> OmniKVMultiStageCache:
         sel = [int(i) for i in self.config.get("do_select_layers").split(",")]
         full = list(range(0, sel[0])) + sel + [self.shape.num_hidden_layers]  # modeling/omnikv.py:322-331
+        if hasattr(self.config, "skip_threshold"):
+            kwargs.setdefault("skip_threshold", self.config.get("skip_threshold"))
         return self.cache_cls(full, self.shape.num_hidden_layers,
                               self.config.get("num_wait_load_layers", 2), self.config.get("real_offload", True), **kwargs)
 

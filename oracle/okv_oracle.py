@@ -268,6 +268,15 @@ def gather_rows(cache: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
     return torch.index_select(cache, 2, idx.view(-1))
 
 
+def idx_overlap_score(new_idx: torch.Tensor, old_idx: torch.Tensor) -> float:
+    """get_idx_iou_score (modeling/spec_cache.py:10-32): the count of indices the two
+    1-D tensors share, divided by the length of the NEW one (the reference's comment
+    says so too: the union is deliberately not used)."""
+    assert new_idx.dim() == 1 and old_idx.dim() == 1
+    un = torch.cat([new_idx, old_idx], dim=0).unique().shape[0]
+    return (new_idx.shape[0] + old_idx.shape[0] - un) / new_idx.shape[0]
+
+
 class OracleMultiStageCache:
     """Plain-torch restatement of OmniKVMultiStageCache
     (modeling/spec_cache.py:253-385), all tensors on the CPU.

@@ -53,13 +53,13 @@ def test_topk_against_golden_ties():
 
 
 # ------------------------------------------------------------------ cache vs oracle cache
-def _run_decode(dtype, real_offload, offload_mode, n=777, steps=3, L=8, sel_layers=(1, 4), wait=1, ratio=0.1):
+def _run_decode(dtype, real_offload, offload_mode, n=777, steps=3, L=8, sel_layers=(1, 4), wait=1, ratio=0.1,
+                cls=OmniKVMultiStageCache):
     hq, hkv, d = 32, 8, 128
     g = torch.Generator().manual_seed(n + L)
     full = orc.full_attn_layers_from_select_layers(list(sel_layers), L)
     ref = orc.OracleMultiStageCache(full, L, wait, real_offload)
-    dut = OmniKVMultiStageCache(full, L, wait, real_offload, max_new_tokens=16, offload_mode=offload_mode,
-                                cpu_num_threads=2)
+    dut = cls(full, L, wait, real_offload, max_new_tokens=16, offload_mode=offload_mode, cpu_num_threads=2)
     kk = orc.num_selected_tokens(ratio, n)
     # prefill
     for i in range(L):
@@ -119,6 +119,60 @@ def test_cache_with_host_offload_tier(dtype, mode):
     for i in sparse:
         assert dut._host_kv[i].is_pinned() and not dut.key_cache[i].is_cuda
     dut._join_worker()
+
+
+@pytest.mark.parametrize("real_offload,mode", [(False, "zero_copy"), (True, "zero_copy"), (True, "memcpy")])
+def test_without_pack_cache_fetches_rows_per_layer(real_offload, mode):
+    """cache_cls `without_pack`: same results as `multi`; with the host tier nothing is
+    staged at selection time, each sparse layer stages its own rows when it runs."""
+    from omnikv_amd.cache import WOPackCache, get_cache_cls
+    from omnikv_amd.config import OmniKVConfig
+    assert get_cache_cls(OmniKVConfig(cache_cls="without_pack")) is WOPackCache
+    staged = []
+    orig = WOPackCache._start_offload
+
+    def spy(self, idx32, layers):
+        staged.append(list(layers))
+        return orig(self, idx32, layers)
+
+    WOPackCache._start_offload = spy
+    try:
+        dut = _run_decode(torch.bfloat16, real_offload=real_offload, offload_mode=mode, cls=WOPackCache)
+    finally:
+        WOPackCache._start_offload = orig
+    if real_offload:
+        assert staged and all(len(l) == 1 for l in staged)  # one layer at a time, never a group
+        dut._join_worker()
+    else:
+        assert staged == []
+
+
+def test_lazy_reselection_skips_similar_selections():
+    """skip_threshold (OmniKVLazyCache.set_out_idx): a selection that overlaps the one in
+    use by more than the threshold is dropped, the rows already staged stay in use."""
+    from omnikv_amd.cache import get_idx_iou_score
+    g = torch.Generator().manual_seed(8)
+    n, kk, L = 600, 60, 4
+    full = orc.full_attn_layers_from_select_layers([0], L)
+    dut = OmniKVMultiStageCache(full, L, 1, False, max_new_tokens=8, skip_threshold=0.5)
+    for i in range(L):
+        dut.update(torch.randn((1, 8, n, 128), generator=g).to(DEV), torch.randn((1, 8, n, 128), generator=g).to(DEV), i)
+    dut.stage = "decoding"
+    a = torch.arange(0, kk, device=DEV)[None]
+    b = torch.cat([torch.arange(0, 40), torch.arange(100, 120)]).to(DEV)[None]   # 40/60 shared: skipped
+    c = torch.cat([torch.arange(0, 20), torch.arange(200, 240)]).to(DEV)[None]   # 20/60 shared: taken
+    assert get_idx_iou_score(b[0], a[0]) == pytest.approx(orc.idx_overlap_score(b[0].cpu(), a[0].cpu()))
+    assert get_idx_iou_score(b[0], a[0]) == pytest.approx(40 / 60)
+    dut.set_idx_on_gpu(a, 0)
+    dut.set_idx_on_gpu(b, 0)
+    assert dut.num_skipped_selections == 1 and torch.equal(dut._idx[0].cpu(), a.cpu().to(torch.int32))
+    dut.set_idx_on_gpu(c, 0)
+    assert dut.num_skipped_selections == 1 and torch.equal(dut._idx[0].cpu(), c.cpu().to(torch.int32))
+    # default: every selection is taken, as the reference's multi-stage cache does
+    ref = OmniKVMultiStageCache(full, L, 1, False)
+    ref.set_idx_on_gpu(a, 0)
+    ref.set_idx_on_gpu(b, 0)
+    assert ref.num_skipped_selections == 0 and torch.equal(ref._idx[0].cpu(), b.cpu().to(torch.int32))
 
 
 def test_offload_stage_packs_rows():

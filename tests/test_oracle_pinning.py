@@ -257,3 +257,19 @@ def test_oracle_cache_against_independent_bookkeeping():
                 assert k_ret.shape[-2] == n + step + 1
                 assert torch.equal(k_ret[:, :, -1:], new_k[i] + step)
     assert cache._seen_tokens == n + 2
+
+
+def test_idx_overlap_score_against_python_sets():
+    """The lazy re-selection score is |new & old| / |new| (not over the union): checked with
+    Python sets on random index lists, and on the closed cases identical / disjoint / nested."""
+    g = torch.Generator().manual_seed(12)
+    for n, k in [(50, 7), (1000, 67), (4096, 274)]:
+        a = torch.randperm(n, generator=g)[:k].sort().values
+        b = torch.randperm(n, generator=g)[:k].sort().values
+        want = len(set(a.tolist()) & set(b.tolist())) / k
+        assert orc.idx_overlap_score(a, b) == pytest.approx(want, abs=1e-12)
+    a = torch.arange(0, 20)
+    assert orc.idx_overlap_score(a, a.clone()) == 1.0
+    assert orc.idx_overlap_score(a, a + 20) == 0.0
+    assert orc.idx_overlap_score(torch.arange(0, 10), torch.arange(0, 40)) == 1.0   # new inside old
+    assert orc.idx_overlap_score(torch.arange(0, 40), torch.arange(0, 10)) == 0.25  # old inside new
