@@ -357,10 +357,7 @@ static void fill_main(RowList* r, const void* k, const void* v, const okv_kv_lay
   r->token_stride = lay->token_stride;
   r->head_stride = lay->head_stride;
   r->batch_stride = lay->batch_stride;
-  r->page_table = lay->page_table;
-  r->page_size = lay->page_size;
-  r->page_table_stride = lay->page_table_stride;
-  r->page_stride = lay->page_stride;
+  rl_set_pages(r, lay->page_table, lay->page_size, lay->page_table_stride, lay->page_stride);
 }
 
 }  // namespace okv

@@ -141,8 +141,8 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
       } else {
         int t = rows.idx ? idx_row[r] : r;
         if (rows.page_table) {
-          tr.row[x] = -1 - (t % rows.page_size);  // slot in page, tagged as paged
-          t = rows.page_table[(int64_t)b * rows.page_table_stride + t / rows.page_size];
+          tr.row[x] = -1 - rl_slot_of(rows, t);  // slot in page, tagged as paged
+          t = rows.page_table[(int64_t)b * rows.page_table_stride + rl_page_of(rows, t)];
         }
         tr.tok[x] = t;
       }
@@ -422,8 +422,8 @@ __global__ __launch_bounds__(1024) void score_raw_mfma(const T* __restrict__ q, 
     r = r < last ? r : last;
     const T* kp;
     if (PAGED) {
-      const int page = rows.page_table[(int64_t)b * rows.page_table_stride + r / rows.page_size];
-      kp = kb + (int64_t)page * rows.page_stride + (uint64_t)(uint32_t)(r % rows.page_size) * ts;
+      const int page = rows.page_table[(int64_t)b * rows.page_table_stride + rl_page_of(rows, r)];
+      kp = kb + (int64_t)page * rows.page_stride + (uint64_t)(uint32_t)rl_slot_of(rows, r) * ts;
     } else {
       kp = kb + (uint64_t)(uint32_t)r * ts;
     }

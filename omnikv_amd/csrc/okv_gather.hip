@@ -58,10 +58,7 @@ int okv_gather_rows(const void* src_base, const okv_kv_layout_t* layout, const i
   r.token_stride = layout->token_stride;
   r.head_stride = layout->head_stride;
   r.batch_stride = layout->batch_stride;
-  r.page_table = layout->page_table;
-  r.page_size = layout->page_size;
-  r.page_table_stride = layout->page_table_stride;
-  r.page_stride = layout->page_stride;
+  rl_set_pages(&r, layout->page_table, layout->page_size, layout->page_table_stride, layout->page_stride);
   r.idx = idx;
   r.idx_stride = idx_stride;
   r.main_lens = sel_lens;

@@ -40,6 +40,7 @@ struct RowList {
   int64_t token_stride, head_stride, batch_stride;  // elements
   const int32_t* page_table;
   int32_t page_size, page_table_stride;
+  int32_t page_shift;  // log2(page_size) when it is a power of two, else -1 (set by rl_set_pages)
   int64_t page_stride;
   const int32_t* idx;  // optional indirection of the main segment
   int64_t idx_stride;
@@ -53,6 +54,26 @@ struct RowList {
   const int32_t* score_lens;  // rows [0, score_len) are scored; 0 = no scoring
   int32_t max_score_len;
 };
+
+// token -> (page slot of its request's table, slot inside the page); shifts when page_size = 2^n
+__device__ __forceinline__ int rl_page_of(const RowList& r, int t) {
+  return r.page_shift >= 0 ? t >> r.page_shift : t / r.page_size;
+}
+__device__ __forceinline__ int rl_slot_of(const RowList& r, int t) {
+  return r.page_shift >= 0 ? t & (r.page_size - 1) : t % r.page_size;
+}
+inline void rl_set_pages(RowList* r, const int32_t* table, int page_size, int table_stride, int64_t page_stride) {
+  r->page_table = table;
+  r->page_size = page_size;
+  r->page_table_stride = table_stride;
+  r->page_stride = page_stride;
+  r->page_shift = -1;
+  if (page_size > 0 && (page_size & (page_size - 1)) == 0) {
+    int sh = 0;
+    while ((1 << sh) < page_size) ++sh;
+    r->page_shift = sh;
+  }
+}
 
 __device__ __forceinline__ int rl_main_len(const RowList& r, int b) {
   return r.main_lens ? r.main_lens[b] : r.max_main_len;
@@ -95,8 +116,8 @@ __device__ __forceinline__ int64_t rl_row_offset(const RowList& r, int b, int ro
   *in_tail = false;
   int t = r.idx ? r.idx[(int64_t)b * r.idx_stride + row] : row;
   if (r.page_table) {
-    int page = r.page_table[(int64_t)b * r.page_table_stride + t / r.page_size];
-    return (int64_t)page * r.page_stride + (int64_t)(t % r.page_size) * r.token_stride;
+    int page = r.page_table[(int64_t)b * r.page_table_stride + rl_page_of(r, t)];
+    return (int64_t)page * r.page_stride + (int64_t)rl_slot_of(r, t) * r.token_stride;
   }
   return (int64_t)b * r.batch_stride + (int64_t)t * r.token_stride;
 }

@@ -25,7 +25,13 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--op", required=True,
                     choices=["dense", "fused", "score", "topk", "sparse", "sparse_packed", "gather", "copy",
-                             "offload_memcpy", "offload_zero_copy", "h2d", "window", "window_loop"])
+                             "offload_memcpy", "offload_zero_copy", "h2d", "window", "window_loop",
+                             "paged_dense", "paged_fused", "paged_score", "paged_topk", "paged_sparse"])
+    ap.add_argument("--batch", type=int, default=16, help="requests of the paged_* ops (ragged lengths 8192..32768)")
+    ap.add_argument("--page-size", type=int, default=16)
+    ap.add_argument("--pages-in-order", action="store_true", help="paged_* ops: identity page table instead of shuffled")
+    ap.add_argument("--contiguous", action="store_true",
+                    help="paged_* ops: the same ragged batch in (bsz, Hkv, Nmax, D) tensors, no page table")
     ap.add_argument("--window", type=int, default=16, help="query positions of the window selectors")
     ap.add_argument("--cpu-threads", type=int, default=8, help="packing threads of the offload tier")
     ap.add_argument("--ctx", type=int, default=131072)
@@ -45,6 +51,8 @@ def main():
     check(lib().okv_set_option(b"split_rows", args.split_rows))
     check(lib().okv_set_option(b"attn_variant", args.attn_variant))
     dev = torch.device("cuda:0")
+    if args.op.startswith("paged_"):
+        return paged(args, dev)
     dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[args.dtype]
     es = 4 if dtype == torch.float32 else 2
     n, tail, nl = args.ctx, args.tail, args.layers
@@ -153,6 +161,82 @@ def main():
     us = e0.elapsed_time(e1) * 1e3 / args.reps
     print(json.dumps({"op": args.op, "ctx": n, "selected": k_sel, "tail": tail, "dtype": args.dtype,
                       "layout": args.layout, "us_per_call": us, "algorithmic_bytes": algo,
+                      "algorithmic_GBps": algo / us / 1e3, "frac_of_8TBps": algo / us / 1e3 / 8000.0}))
+
+
+def paged(args, dev):
+    """The batched serving shape: `--batch` requests of ragged length in one paged pool
+    (pages shuffled from a seed), per-request k = int(ratio * length)."""
+    dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[args.dtype]
+    es = 4 if dtype == torch.float32 else 2
+    lens = synth.ragged_lengths(args.batch)
+    table, total = synth.shuffled_page_table(lens, args.page_size)
+    if args.pages_in_order:
+        flat = torch.sort(table.flatten()[table.flatten() >= 0]).values  # same pages, ascending per request
+        pages = [(int(l) + args.page_size - 1) // args.page_size for l in lens]
+        o = 0
+        for b, pcount in enumerate(pages):
+            table[b, :pcount] = torch.arange(o, o + pcount, dtype=torch.int32)
+            o += pcount
+    gen = torch.Generator(device=dev).manual_seed(11)
+    nl = args.layers
+    pools = []
+    for _ in range(nl):
+        if args.contiguous:
+            nmax_ = int(lens.max())
+            pools.append((torch.empty((args.batch, HKV, nmax_, D), dtype=dtype, device=dev).normal_(generator=gen),
+                          torch.empty((args.batch, HKV, nmax_, D), dtype=dtype, device=dev).normal_(generator=gen)))
+            continue
+        pk = torch.empty((total, args.page_size, HKV, D), dtype=dtype, device=dev).normal_(generator=gen)
+        pv = torch.empty((total, args.page_size, HKV, D), dtype=dtype, device=dev).normal_(generator=gen)
+        pools.append(ops.PagedKV(pk, pv, table.to(dev), args.page_size))
+    if args.contiguous:
+        dense_ = lambda q, kv, **kw: ops.dense_attn(q, kv[0], kv[1], **kw)
+        sparse_ = lambda q, kv, **kw: ops.sparse_attn(q, kv[0], kv[1], **kw)
+        score_ = lambda q, kv, **kw: ops.score(q, kv[0], **kw)
+    else:
+        dense_, sparse_, score_ = ops.dense_attn, ops.sparse_attn, ops.score
+    qs = [torch.randn((args.batch, HQ, 1, D), generator=gen, device=dev).to(dtype) for _ in range(nl)]
+    lens_d = lens.to(dev)
+    nmax = int(lens.max())
+    k_per = torch.tensor([max(1, int(args.ratio * int(n))) for n in lens], dtype=torch.int32)
+    kmax, k_per_d = int(k_per.max()), k_per.to(dev)
+    _, scores = dense_(qs[0], pools[0], seq_len=nmax, seq_lens=lens_d, selector=args.selector, score_len=nmax,
+                               score_lens=lens_d)
+    idx = torch.zeros((args.batch, kmax), dtype=torch.int32, device=dev)
+    ops.topk(scores, kmax, seq_lens=lens_d, k_per_seg=k_per_d, out=idx)
+
+    def call(i):
+        l = i % nl
+        if args.op == "paged_dense":
+            return dense_(qs[l], pools[l], seq_len=nmax, seq_lens=lens_d)
+        if args.op == "paged_fused":
+            return dense_(qs[l], pools[l], seq_len=nmax, seq_lens=lens_d, selector=args.selector,
+                                  score_len=nmax, score_lens=lens_d)
+        if args.op == "paged_score":
+            return score_(qs[l], pools[l], score_len=nmax, selector=args.selector, score_lens=lens_d)
+        if args.op == "paged_topk":
+            return ops.topk(scores, kmax, seq_lens=lens_d, k_per_seg=k_per_d, out=idx)
+        return sparse_(qs[l], pools[l], idx=idx, sel_len=kmax, sel_lens=k_per_d)
+
+    tokens, sel = int(lens.sum()), int(k_per.sum())
+    row = HKV * D * es
+    algo = {"paged_dense": 2.0 * tokens * row, "paged_fused": 2.0 * tokens * row + 4.0 * tokens,
+            "paged_score": 1.0 * tokens * row + 4.0 * tokens, "paged_topk": 4.0 * tokens + 4.0 * sel,
+            "paged_sparse": 2.0 * sel * row + 4.0 * sel}[args.op]
+    for i in range(args.warmup):
+        call(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    stream = torch.cuda.current_stream()
+    e0.record(stream)
+    for i in range(args.reps):
+        call(i)
+    e1.record(stream)
+    e1.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / args.reps
+    print(json.dumps({"op": args.op, "batch": args.batch, "page_size": args.page_size, "tokens": tokens,
+                      "selected": sel, "dtype": args.dtype, "us_per_call": us, "algorithmic_bytes": algo,
                       "algorithmic_GBps": algo / us / 1e3, "frac_of_8TBps": algo / us / 1e3 / 8000.0}))
 
 
