@@ -81,7 +81,8 @@ __host__ __device__ constexpr int stage1_lds_floats(bool with_v) {
 }
 
 // MODE 0: contiguous rows, no index, no tail.  MODE 1: rows through idx (no page table),
-// optional tail.  MODE 2: anything (page tables, idx or not, tail or not).
+// optional tail.  MODE 2: anything (page tables, idx or not, tail or not).  MODE 3: page
+// table with pages of 2^n >= 16 rows, no index, no tail (a tile never straddles a page).
 template <typename T, int G, bool WITH_V, int MODE, bool LOGITS>
 __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q, RowList rows,
                                                         int hq, float scale, AttnWorkspace w) {
@@ -132,6 +133,10 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
       tr.row[x] = r;
       if (MODE == 0) {
         tr.tok[x] = r;
+      } else if (MODE == 3) {
+        // pages of 16k rows: the whole tile lies in one page, looked up once through the scalar unit
+        const int tb = __builtin_amdgcn_readfirstlane(tbase);
+        tr.tok[x] = rows.page_table[(int64_t)b * rows.page_table_stride + (tb >> rows.page_shift)];
       } else if (MODE == 1) {  // branch-free: main_len >= 1 is guaranteed by the launcher
         const int ri = r < main_len ? r : main_len - 1;
         const int t = idx_row[ri];
@@ -150,6 +155,9 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
   };
   auto row_ptr = [&](const TileRows& tr, int x, bool is_v) -> const T* {
     if (MODE == 0) return (is_v ? vb : kb) + (uint64_t)(uint32_t)tr.tok[x] * ts;
+    if (MODE == 3)
+      return (is_v ? pvb : pkb) + (int64_t)tr.tok[x] * rows.page_stride +
+             (uint64_t)(uint32_t)(tr.row[x] & (rows.page_size - 1)) * ts;
     if (MODE == 1) {
       const bool in_tail = tr.row[x] >= main_len;
       const T* base = in_tail ? (is_v ? tvb : tkb) : (is_v ? vb : kb);
@@ -358,10 +366,12 @@ static void launch_g(const void* q, const RowList& rows, int hq, int hkv, int ba
   int mode = 2;
   if (!rows.idx && !rows.page_table && no_tail) mode = 0;
   else if (rows.idx && !rows.page_table && !rows.main_lens && rows.max_main_len >= 1) mode = 1;
+  else if (rows.page_table && !rows.idx && no_tail && rows.page_shift >= 4) mode = 3;
 #define OKV_MODES(WV, LG)                                                                  \
   do {                                                                                     \
     if (mode == 0) launch_one<T, G, WV, 0, LG>(q, rows, hq, hkv, batch, scale, w, stream); \
     else if (mode == 1) launch_one<T, G, WV, 1, LG>(q, rows, hq, hkv, batch, scale, w, stream); \
+    else if (mode == 3) launch_one<T, G, WV, 3, LG>(q, rows, hq, hkv, batch, scale, w, stream); \
     else launch_one<T, G, WV, 2, LG>(q, rows, hq, hkv, batch, scale, w, stream);           \
   } while (0)
   if (!with_v) OKV_MODES(false, true);  // scoring only
@@ -422,7 +432,11 @@ __global__ __launch_bounds__(1024) void score_raw_mfma(const T* __restrict__ q, 
     r = r < last ? r : last;
     const T* kp;
     if (PAGED) {
-      const int page = rows.page_table[(int64_t)b * rows.page_table_stride + rl_page_of(rows, r)];
+      // pages of 2^n >= 16 rows hold the whole tile: one lookup through the scalar unit
+      const int page = rows.page_shift >= 4
+                           ? rows.page_table[(int64_t)b * rows.page_table_stride +
+                                             (__builtin_amdgcn_readfirstlane(tbase) >> rows.page_shift)]
+                           : rows.page_table[(int64_t)b * rows.page_table_stride + rl_page_of(rows, r)];
       kp = kb + (int64_t)page * rows.page_stride + (uint64_t)(uint32_t)rl_slot_of(rows, r) * ts;
     } else {
       kp = kb + (uint64_t)(uint32_t)r * ts;
@@ -492,8 +506,10 @@ static void launch_score_raw_g(const void* q, const RowList& rows, int hq, int h
     int n = 0;
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
   }
-  // one round of workgroups, three resident per CU, equal shares of the rows
-  int64_t per = ((int64_t)rows.max_score_len * batch + (int64_t)cus * 3 - 1) / ((int64_t)cus * 3);
+  // one round of workgroups, three resident per CU, equal shares of the rows; a batch may be
+  // ragged (short requests leave their blocks empty), so it gets blocks half the size
+  const int64_t slots = (int64_t)cus * (batch > 1 ? 6 : 3);
+  int64_t per = ((int64_t)rows.max_score_len * batch + slots - 1) / slots;
   int rpb = (int)((per + 15) / 16 * 16);
   if (rpb < 64) rpb = 64;
   if (rpb > 1024) rpb = 1024;
