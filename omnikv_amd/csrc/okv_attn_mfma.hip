@@ -80,6 +80,11 @@ __host__ __device__ constexpr int stage1_lds_floats(bool with_v) {
   return 3 * 16 * G + 16 + (with_v ? 16 * G * kD : 0);
 }
 
+// The streaming modes (0, 3) load K as whole rows and transpose the tile in LDS (see
+// k_rows_to_a_operand); the gather modes keep the direct A-operand loads: their pass is a
+// chain of latencies and the detour adds to it (measured: 13.5 vs 13.1 us at 8781 rows).
+__host__ __device__ constexpr bool stage1_k_through_lds(int mode) { return mode == 0 || mode == 3; }
+
 // MODE 0: contiguous rows, no index, no tail.  MODE 1: rows through idx (no page table),
 // optional tail.  MODE 2: anything (page tables, idx or not, tail or not).  MODE 3: page
 // table with pages of 2^n >= 16 rows, no index, no tail (a tile never straddles a page).
@@ -87,6 +92,7 @@ template <typename T, int G, bool WITH_V, int MODE, bool LOGITS>
 __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q, RowList rows,
                                                         int hq, float scale, AttnWorkspace w) {
   extern __shared__ float lds[];
+  constexpr bool KLDS = stage1_k_through_lds(MODE);
   const int g = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
   const int main_len = rl_main_len(rows, b);
   const int L = main_len + rl_tail_len(rows, b);
@@ -170,13 +176,22 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
     return (is_v ? vb : kb) + (uint64_t)(uint32_t)tr.tok[x] * ts;
   };
   auto load_tile = [&](const TileRows& tr, uint4 (&kf)[4], uint4 (&vf)[4]) {
-    const T* kp = row_ptr(tr, 0, false) + 8 * j4;
+    if (KLDS) {
+      // whole rows, like V; compute() turns the tile into the A-operand layout through LDS
 #pragma unroll
-    for (int s = 0; s < 4; ++s) kf[s] = *reinterpret_cast<const uint4*>(kp + 32 * s);
+      for (int i = 0; i < 4; ++i) kf[i] = load_stream16(row_ptr(tr, 1 + i, false) + 8 * r16);
+    } else {
+      const T* kp = row_ptr(tr, 0, false) + 8 * j4;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) kf[s] = *reinterpret_cast<const uint4*>(kp + 32 * s);
+    }
     if (WITH_V) {
+      // V rows are consumed whole (256 bytes per 16 lanes) and never read again in this launch:
+      // streamed.  K in the direct layout is not: a row's 128-byte lines are consumed by two
+      // consecutive loads, and a streamed line can leave L1 between them (measured: slower).
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        vf[i] = *reinterpret_cast<const uint4*>(row_ptr(tr, 1 + i, true) + 8 * r16);
+        vf[i] = load_stream16(row_ptr(tr, 1 + i, true) + 8 * r16);
     }
   };
 
@@ -190,7 +205,18 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
   const bool scored = LOGITS && begin < A;  // a scored split ends at or before A
   float* slog = lds;  // [G][split_rows] scaled logits of the split; flushed before LDS is reused below
 
-  auto compute = [&](int tbase, const uint4 (&kf)[4], const uint4 (&vf)[4]) {
+  // K staging of the streaming modes: 4 KB per wave behind everything else the block keeps in LDS
+  int kst_off = stage1_lds_floats<G>(WITH_V);
+  if (LOGITS && G * w.split_rows > kst_off) kst_off = G * w.split_rows;
+  char* kstage = reinterpret_cast<char*>(lds + kst_off) + wave * 4096;
+  auto compute = [&](int tbase, const uint4 (&kf_in)[4], const uint4 (&vf)[4]) {
+    uint4 kf[4];
+    if (KLDS) {
+      k_rows_to_a_operand(kstage, r16, j4, kf_in, kf);
+    } else {
+#pragma unroll
+      for (int s = 0; s < 4; ++s) kf[s] = kf_in[s];
+    }
     f32x4_t S = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < 4; ++s) S = mfma16((const T*)nullptr, kf[s], qf[s], S);
@@ -348,6 +374,7 @@ static void launch_one(const void* q, const RowList& rows, int hq, int hkv, int 
   auto kern = attn_stage1_mfma<T, G, WITH_V, MODE, LOGITS>;
   size_t lds_floats = stage1_lds_floats<G>(WITH_V);  // the logits staging aliases the merge buffers
   if (LOGITS && (size_t)G * w.split_rows > lds_floats) lds_floats = (size_t)G * w.split_rows;
+  if (stage1_k_through_lds(MODE)) lds_floats += 4 * 1024;  // 4 KB of K staging per wave
   const size_t lds_bytes = lds_floats * sizeof(float);
   static size_t configured = 0;
   if (lds_bytes > configured) {
@@ -403,7 +430,7 @@ __global__ __launch_bounds__(1024) void score_raw_mfma(const T* __restrict__ q, 
                                                        float scale, int head_reduce,
                                                        int rows_per_block, float* __restrict__ scores,
                                                        int64_t score_stride) {
-  extern __shared__ float lds[];  // [kv heads][rows_per_block]
+  extern __shared__ float lds[];  // [kv heads][rows_per_block] scores, then 4 KB of K staging per wave
   const int b = blockIdx.y;
   const int A = rl_score_len(rows, b);
   const int begin = blockIdx.x * rows_per_block;
@@ -423,29 +450,35 @@ __global__ __launch_bounds__(1024) void score_raw_mfma(const T* __restrict__ q, 
       qf[s] = r16 < G ? v : make_uint4(0, 0, 0, 0);
     }
   }
-  const T* kb = reinterpret_cast<const T*>(rows.k_base) + (int64_t)g * rows.head_stride + 8 * j4 +
+  const T* kb = reinterpret_cast<const T*>(rows.k_base) + (int64_t)g * rows.head_stride + 8 * r16 +
                 (PAGED ? 0 : (int64_t)b * rows.batch_stride);
   const uint32_t ts = (uint32_t)rows.token_stride;
   const int last = end - 1;
+  // whole rows (instruction i: rows 4*(l/16) + i), transposed for the matrix cores in compute()
   auto load_tile = [&](int tbase, uint4 (&kf)[4]) {
-    int r = tbase + r16;
-    r = r < last ? r : last;
-    const T* kp;
-    if (PAGED) {
-      // pages of 2^n >= 16 rows hold the whole tile: one lookup through the scalar unit
-      const int page = rows.page_shift >= 4
-                           ? rows.page_table[(int64_t)b * rows.page_table_stride +
-                                             (__builtin_amdgcn_readfirstlane(tbase) >> rows.page_shift)]
-                           : rows.page_table[(int64_t)b * rows.page_table_stride + rl_page_of(rows, r)];
-      kp = kb + (int64_t)page * rows.page_stride + (uint64_t)(uint32_t)rl_slot_of(rows, r) * ts;
-    } else {
-      kp = kb + (uint64_t)(uint32_t)r * ts;
-    }
+    int page = 0;
+    if (PAGED && rows.page_shift >= 4)  // pages of 2^n >= 16 rows hold the whole tile: one scalar lookup
+      page = rows.page_table[(int64_t)b * rows.page_table_stride +
+                             (__builtin_amdgcn_readfirstlane(tbase) >> rows.page_shift)];
 #pragma unroll
-    for (int s = 0; s < 4; ++s) kf[s] = *reinterpret_cast<const uint4*>(kp + 32 * s);
+    for (int i = 0; i < 4; ++i) {
+      int r = tbase + 4 * j4 + i;
+      r = r < last ? r : last;
+      const T* kp;
+      if (PAGED) {
+        if (rows.page_shift < 4) page = rows.page_table[(int64_t)b * rows.page_table_stride + rl_page_of(rows, r)];
+        kp = kb + (int64_t)page * rows.page_stride + (uint64_t)(uint32_t)rl_slot_of(rows, r) * ts;
+      } else {
+        kp = kb + (uint64_t)(uint32_t)r * ts;
+      }
+      kf[i] = load_stream16(kp);
+    }
   };
+  char* kstage = reinterpret_cast<char*>(lds + (blockDim.x >> 6) * rows_per_block) + g * 4096;
   float* mine = lds + g * rows_per_block;
-  auto compute = [&](int tbase, const uint4 (&kf)[4]) {
+  auto compute = [&](int tbase, const uint4 (&kf_in)[4]) {
+    uint4 kf[4];
+    k_rows_to_a_operand(kstage, r16, j4, kf_in, kf);
     f32x4_t S = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < 4; ++s) S = mfma16((const T*)nullptr, kf[s], qf[s], S);
@@ -514,13 +547,22 @@ static void launch_score_raw_g(const void* q, const RowList& rows, int hq, int h
   if (rpb < 64) rpb = 64;
   if (rpb > 1024) rpb = 1024;
   dim3 grid((rows.max_score_len + rpb - 1) / rpb, batch), block(64 * hkv);
-  const size_t lds_bytes = (size_t)hkv * rpb * sizeof(float);
-  if (rows.page_table)
-    hipLaunchKernelGGL((score_raw_mfma<T, G, true>), grid, block, lds_bytes, stream, (const T*)q, rows, hq,
-                       scale, head_reduce, rpb, scores, score_stride);
-  else
-    hipLaunchKernelGGL((score_raw_mfma<T, G, false>), grid, block, lds_bytes, stream, (const T*)q, rows,
-                       hq, scale, head_reduce, rpb, scores, score_stride);
+  const size_t lds_bytes = (size_t)hkv * rpb * sizeof(float) + (size_t)hkv * 4096;  // scores + K staging
+  if (rows.page_table) {
+    auto kern = score_raw_mfma<T, G, true>;
+    if (lds_bytes > 48 * 1024)
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds_bytes);
+    hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const T*)q, rows, hq, scale, head_reduce, rpb,
+                       scores, score_stride);
+  } else {
+    auto kern = score_raw_mfma<T, G, false>;
+    if (lds_bytes > 48 * 1024)
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds_bytes);
+    hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const T*)q, rows, hq, scale, head_reduce, rpb,
+                       scores, score_stride);
+  }
 }
 
 template <typename T>

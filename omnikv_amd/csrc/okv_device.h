@@ -86,4 +86,34 @@ __device__ __forceinline__ f32x4_t mfma16(const F16*, const uint4& a, const uint
   return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
                                                 __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
 }
+
+// ---- K tiles for the matrix cores, loaded as whole rows.
+// A 16-byte load per lane straight into the A-operand layout touches 16 different rows per
+// 16 lanes (64 bytes of each); loading like V instead -- instruction i brings rows
+// 4*(l/16) + i, lane l%16 its 16-byte chunk, whole 256-byte rows per 16 lanes, marked
+// non-temporal -- streams measurably faster, and the tile is turned into the A-operand layout
+// through a wave-private 4 KB of LDS: row R at R*256, its chunk c at position c ^ R, so the
+// 16 lanes that write a row and the 16 lanes that read one k-chunk of 16 rows both cover all
+// banks exactly once.  The LDS operations of one wave execute in order: no s_barrier.
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+__device__ __forceinline__ uint4 load_stream16(const void* p) {
+  const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void k_rows_to_a_operand(char* stage, int r16, int j4, const uint4 (&rows_in)[4],
+                                                    uint4 (&a)[4]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int R = 4 * j4 + i;
+    *reinterpret_cast<uint4*>(stage + R * 256 + 16 * (r16 ^ R)) = rows_in[i];
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int s = 0; s < 4; ++s)
+    a[s] = *reinterpret_cast<const uint4*>(stage + r16 * 256 + 16 * ((4 * s + j4) ^ r16));
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();  // the next tile's writes stay behind these reads
+}
 }  // namespace okv
