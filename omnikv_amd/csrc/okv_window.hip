@@ -66,7 +66,6 @@ __device__ __forceinline__ void load_window_q(const WindowArgs& a, int b, int g,
 template <typename T, int NCB>
 __global__ __launch_bounds__(256) void window_lse_mfma(WindowArgs a) {
   __shared__ float sm[16][16 * NCB], sl[16][16 * NCB];
-  __shared__ __attribute__((aligned(16))) char kst[4][4096];  // K staging, one tile per wave
   const int g = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
   const int A = win_len(a, b);
   const int begin = split * a.split_rows;
@@ -78,19 +77,20 @@ __global__ __launch_bounds__(256) void window_lse_mfma(WindowArgs a) {
   uint4 qf[NCB][4];
   load_window_q<T, NCB>(a, b, g, r16, j4, qf);
   const T* kb = reinterpret_cast<const T*>(a.k_base) + (int64_t)b * a.batch_stride +
-                (int64_t)g * a.head_stride + 8 * r16;
+                (int64_t)g * a.head_stride + 8 * j4;
   const uint32_t ts = (uint32_t)a.token_stride;
   const int last = end - 1;
-  // whole rows (instruction i: rows 4*(l/16) + i), transposed for the matrix cores in compute()
+  // K straight into the A-operand layout with ordinary (cached) loads in both passes.  Measured
+  // alternatives: whole rows streamed (non-temporal) and transposed through LDS make pass 1 no
+  // faster and pass 2 slower (78 vs 69 us: streamed lines do not stay in the memory-side cache
+  // for the second reading); in pass 2 the LDS detour waits on the LDS atomics (128 us).
   auto load_tile = [&](int tbase, uint4 (&kf)[4]) {
+    int r = tbase + r16;
+    r = r < last ? r : last;
+    const T* kp = kb + (uint64_t)(uint32_t)r * ts;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      int r = tbase + 4 * j4 + i;
-      r = r < last ? r : last;
-      kf[i] = load_stream16(kb + (uint64_t)(uint32_t)r * ts);
-    }
+    for (int s = 0; s < 4; ++s) kf[s] = *reinterpret_cast<const uint4*>(kp + 32 * s);
   };
-  char* kstage = kst[wave];
   const float sl2 = a.scale * kLog2e;
   float m[NCB], l[NCB];  // per column block: state of (column r16, lane row j4), m in raw units
 #pragma unroll
@@ -98,10 +98,8 @@ __global__ __launch_bounds__(256) void window_lse_mfma(WindowArgs a) {
     m[cb] = -INFINITY;
     l[cb] = 0.f;
   }
-  auto compute = [&](int tbase, const uint4 (&kf_in)[4]) {
+  auto compute = [&](int tbase, const uint4 (&kf)[4]) {
     const int row0 = tbase + 4 * j4;
-    uint4 kf[4];
-    k_rows_to_a_operand(kstage, r16, j4, kf_in, kf);
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) {
       f32x4_t S = {0.f, 0.f, 0.f, 0.f};
@@ -241,8 +239,6 @@ __global__ __launch_bounds__(512) void window_score_mfma(WindowArgs a, int rows_
                 (int64_t)g * a.head_stride + 8 * j4;
   const uint32_t ts = (uint32_t)a.token_stride;
   const int last = end - 1;
-  // straight into the A-operand layout: a detour through LDS (as pass 1 takes) would wait on
-  // the LDS atomics of the previous tile, which this way stay off the critical path
   auto load_tile = [&](int tbase, uint4 (&kf)[4]) {
     int r = tbase + r16;
     r = r < last ? r : last;
