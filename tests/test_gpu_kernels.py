@@ -346,3 +346,31 @@ def test_window_unsupported_shapes_are_refused():
     assert not ops.window_supported(q32.to(DEV), k32.to(DEV))
     with pytest.raises(Exception, match="unsupported"):
         ops.score_window(q32.to(DEV), k32.to(DEV), selector="uniform")
+
+
+# ------------------------------------------------------------------ other GQA group sizes
+@pytest.mark.parametrize("hq,hkv", [(8, 8), (16, 8), (64, 8), (4, 1), (32, 4)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_group_sizes_one_two_eight(hq, hkv, dtype):
+    """Groups of 1, 2 and 8 q heads per kv head (the benchmark geometry is 4): dense with fused
+    scores, raw scoring, top-k and the sparse pass against the oracle."""
+    n, tail, kk = 3001, 3, 200
+    g = torch.Generator().manual_seed(hq * 100 + hkv)
+    q = torch.randn((1, hq, 1, 128), generator=g).to(dtype)
+    k = torch.randn((1, hkv, n + tail, 128), generator=g).to(dtype)
+    v = torch.randn((1, hkv, n + tail, 128), generator=g).to(dtype)
+    k[:, :, 0] *= 6
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
+    out, sc = ops.dense_attn(q.to(DEV), k.to(DEV), v.to(DEV), selector="softmax_before_last", score_len=n)
+    assert (out.cpu().float() - orc.gqa_attention(q.float(), k.float(), v.float())[:, :, 0]).abs().max() < tol
+    want = orc.score_tokens(q.float(), k.float(), n, "softmax_before_last")
+    assert _rel_err(sc.cpu(), want) < 1e-4
+    raw = ops.score(q.to(DEV), k.to(DEV)[:, :, :n], selector="last")
+    assert _rel_err(raw.cpu(), orc.score_tokens(q.float(), k.float(), n, "last")) < 1e-4
+    idx = ops.topk(sc, kk)
+    assert torch.equal(idx.cpu().to(torch.int64), orc.select_topk_stable(sc.cpu(), kk))
+    sp = ops.sparse_attn(q.to(DEV), k.to(DEV)[:, :, :n], v.to(DEV)[:, :, :n], idx=idx,
+                         tail_k=k.to(DEV)[:, :, n:], tail_v=v.to(DEV)[:, :, n:])
+    ks = torch.cat([orc.gather_rows(k[:, :, :n], idx.cpu().to(torch.int64)), k[:, :, n:]], dim=2)
+    vs = torch.cat([orc.gather_rows(v[:, :, :n], idx.cpu().to(torch.int64)), v[:, :, n:]], dim=2)
+    assert (sp.cpu().float() - orc.gqa_attention(q.float(), ks.float(), vs.float())[:, :, 0]).abs().max() < tol

@@ -32,7 +32,7 @@ def _paged_batch(lens, page_size, dtype, seed=0):
     return q, ks, vs, pool_k, pool_v, table
 
 
-@pytest.mark.parametrize("page_size", [1, 16])
+@pytest.mark.parametrize("page_size", [1, 8, 12, 16, 64])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_paged_ragged_batch(page_size, dtype):
     lens = torch.tensor([700, 33, 1500, 1, 16, 1024, 257], dtype=torch.int32)
