@@ -167,22 +167,29 @@ class OmniKVMultiStageCache:
         shape, so that a whole decode step can be captured in a HIP graph and replayed.
         Sequence lengths and append positions become device scalars (the kernels read
         per-request lengths from device memory); every buffer a step touches is
-        preallocated.  Not available with real_offload (its staging needs the host)."""
-        if self.real_offload:
-            raise NotImplementedError("static decode keeps every layer on the GPU (real_offload=False)")
+        preallocated.  With real_offload only the zero-copy mode qualifies: there the GPU
+        fetches the selected pinned rows itself, on the copy stream, and the fork and join of
+        that stream become part of the graph; the memcpy mode packs rows on host threads."""
+        if self.real_offload and self.offload_mode != "zero_copy":
+            raise NotImplementedError("static decode with real_offload needs offload_mode='zero_copy'")
         if self._static:
             return
         any_store = next(iter(self._store.values()))
         dev = any_store.k.device
         n = self._seen_tokens
+        self._finish_prefill_offload()
         for layer_idx, sparse in ((i, s[0]) for i, s in self.layer_state.items()):
-            st = self._store[layer_idx]
             if sparse:
                 if layer_idx not in self._tail:
-                    b, hkv, _, d = st.k.shape
-                    self._tail[layer_idx] = _Store(b, self.max_new_tokens, hkv, d, st.k.dtype, dev)
+                    if self.real_offload:
+                        host = self._host_kv[layer_idx]
+                        b, hkv, d, dt = 1, host.shape[2], host.shape[3], host.dtype
+                    else:
+                        st = self._store[layer_idx]
+                        (b, hkv, _, d), dt = st.k.shape, st.k.dtype
+                    self._tail[layer_idx] = _Store(b, self.max_new_tokens, hkv, d, dt, dev)
             else:
-                st.reserve(n + self.max_new_tokens)
+                self._store[layer_idx].reserve(n + self.max_new_tokens)
         tails = [t.len for t in self._tail.values()]
         t0 = tails[0] if tails else 0
         self._pos = torch.tensor([n], dtype=torch.int64, device=dev)
@@ -363,6 +370,31 @@ class OmniKVMultiStageCache:
         self._worker = threading.Thread(target=work, daemon=True)
         self._worker.start()
 
+    def _stage_static(self, sel_layer_idx: int, idx32: torch.Tensor) -> None:
+        """Static decode with the host tier: the copy stream gathers the selected pinned rows
+        of every layer of the group (the GPU reads host memory itself), one event per layer.
+        Nothing here touches the host, so the whole exchange is captured with the step."""
+        hi = self.layer_state[sel_layer_idx][2]
+        lo = sel_layer_idx + self.num_wait_layers + 1
+        if lo >= hi:
+            return
+        dev, k = idx32.device, idx32.shape[1]
+        if self._copy_stream is None:
+            self._copy_stream = torch.cuda.Stream(device=dev)
+        self._copy_stream.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(self._copy_stream):
+            for i in range(lo, hi):
+                host = self._host_kv[i]
+                part = self._part.get(i)
+                if part is None or part.shape[1] != k:
+                    part = torch.empty((1, k) + tuple(host.shape[1:]), dtype=host.dtype, device=dev)
+                    self._part[i] = part
+                if i not in self._events:
+                    self._events[i] = torch.cuda.Event()
+                _gather_wide(host.view(1, host.shape[0], 1, -1).permute(0, 2, 1, 3), idx32,
+                             part.view(1, k, 1, -1).permute(0, 2, 1, 3))
+                self._events[i].record(self._copy_stream)
+
     def _join_worker(self):
         if self._worker is not None:
             self._worker.join()
@@ -404,6 +436,13 @@ class OmniKVMultiStageCache:
         """Decode attention of `layer_idx` over what update() would have returned,
         without building it.  query_states: (bsz, Hq, 1, D); returns (bsz, Hq, D)."""
         if self._static:
+            if self.layer_state[layer_idx][0] and self.real_offload:
+                # rows staged by the copy stream since the filter layer ran (_stage_static)
+                torch.cuda.current_stream(query_states.device).wait_event(self._events[layer_idx])
+                part, tl = self._part[layer_idx], self._tail[layer_idx]
+                return ops.sparse_attn(query_states, part[:, :, 0].permute(0, 2, 1, 3), part[:, :, 1].permute(0, 2, 1, 3),
+                                       tail_k=tl.k, tail_v=tl.v, tail_len=tl.capacity, tail_lens=self._tail_len32,
+                                       scale=scale)
             st = self._store[layer_idx]
             if self.layer_state[layer_idx][0]:
                 tl = self._tail[layer_idx]
@@ -441,6 +480,8 @@ class OmniKVMultiStageCache:
                 buf = torch.empty((scores.shape[0], k), dtype=torch.int32, device=scores.device)
                 self._idx[layer_idx] = buf  # the sparse layers keep reading this very buffer
             ops.topk(scores, k, out=buf)
+            if self.real_offload:
+                self._stage_static(layer_idx, buf)
             return out, buf
         kview, vview = self._store[layer_idx].views()
         out, scores = ops.dense_attn(query_states, kview, vview, selector=selector_cls, score_len=consider_len,

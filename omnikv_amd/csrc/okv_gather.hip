@@ -9,7 +9,7 @@
 
 namespace okv {
 
-// One thread moves 16 bytes.  grid (ceil(units/256), batch).
+// One thread moves 16 bytes at a time, grid-stride.  grid (blocks, batch).
 __global__ __launch_bounds__(256) void gather_rows_kernel(RowList rows, int hkv, int esize,
                                                           char* __restrict__ dst,
                                                           int64_t dst_token_stride,
@@ -18,18 +18,19 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(RowList rows, int hkv,
   const int b = blockIdx.y;
   const int n = rl_main_len(rows, b);
   const int upr = kHeadDimBytes16(esize);
-  const int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int per_token = hkv * upr;
-  const int64_t j = u / per_token;
-  if (j >= n) return;
-  const int rem = (int)(u % per_token);
-  const int g = rem / upr, x = rem % upr;
-  bool in_tail;
-  int64_t so = rl_row_offset(rows, b, (int)j, n, &in_tail) + (int64_t)g * rows.head_stride;
-  int64_t dofs = (int64_t)b * dst_batch_stride + j * dst_token_stride + (int64_t)g * dst_head_stride;
-  const uint4* sp = reinterpret_cast<const uint4*>((const char*)rows.k_base + so * esize) + x;
-  uint4* dp = reinterpret_cast<uint4*>(dst + dofs * esize) + x;
-  *dp = *sp;
+  const int64_t units = (int64_t)n * per_token;
+  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < units; u += (int64_t)gridDim.x * 256) {
+    const int64_t j = u / per_token;
+    const int rem = (int)(u % per_token);
+    const int g = rem / upr, x = rem % upr;
+    bool in_tail;
+    int64_t so = rl_row_offset(rows, b, (int)j, n, &in_tail) + (int64_t)g * rows.head_stride;
+    int64_t dofs = (int64_t)b * dst_batch_stride + j * dst_token_stride + (int64_t)g * dst_head_stride;
+    const uint4* sp = reinterpret_cast<const uint4*>((const char*)rows.k_base + so * esize) + x;
+    uint4* dp = reinterpret_cast<uint4*>(dst + dofs * esize) + x;
+    *dp = *sp;
+  }
 }
 
 }  // namespace okv
@@ -64,7 +65,17 @@ int okv_gather_rows(const void* src_base, const okv_kv_layout_t* layout, const i
   r.main_lens = sel_lens;
   r.max_main_len = max_sel_len;
   const int64_t units = (int64_t)max_sel_len * layout->num_kv_heads * kHeadDimBytes16(esize);
-  dim3 grid((unsigned)((units + 255) / 256), batch);
+  int64_t blocks = (units + 255) / 256;
+  // A source in host memory (the zero-copy offload tier) is read over the host link: a few
+  // waves with loads in flight saturate it, and a grid of the usual size would sit on every
+  // CU's wave slots waiting for the link while the kernels of the other streams starve.
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, src_base) == hipSuccess) {
+    if (attr.type == hipMemoryTypeHost && blocks > 64) blocks = 64;
+  } else {
+    (void)hipGetLastError();  // unregistered pointer: not ours to judge
+  }
+  dim3 grid((unsigned)blocks, batch);
   hipLaunchKernelGGL(gather_rows_kernel, grid, dim3(256), 0, (hipStream_t)stream, r,
                      layout->num_kv_heads, esize, (char*)dst, dst_token_stride, dst_head_stride,
                      dst_batch_stride);

@@ -140,16 +140,16 @@ def test_generate_greedy_and_error_paths():
         lm2.forward(ids[:, :1], cache)
 
 
-@pytest.mark.parametrize("selector_cls", ["last", "softmax_before_last"])
-def test_graph_replayed_decode_matches_eager(selector_cls):
-    """A decode step captured in a HIP graph (device-side lengths and positions) must
-    reproduce the eager path token for token and logit for logit on every replay."""
-    cfg = _config(selector_cls, False)
+@pytest.mark.parametrize("selector_cls,offload", [("last", False), ("softmax_before_last", False), ("last", True)])
+def test_graph_replayed_decode_matches_eager(selector_cls, offload):
+    """A decode step captured in a HIP graph (device-side lengths and positions; with the
+    host tier also the copy stream's zero-copy gathers) must reproduce the eager path
+    token for token and logit for logit on every replay."""
     ids = torch.randint(0, SHAPE.vocab_size, (1, 400), generator=torch.Generator().manual_seed(4)).to(DEV)
     steps = 7
 
     def fresh():
-        lm = OmniKVMulLM(SHAPE, _config(selector_cls, False)).float().to(DEV)
+        lm = OmniKVMulLM(SHAPE, _config(selector_cls, offload)).float().to(DEV)
         lm.init_weights(seed=11, std=0.08)
         return lm
 
@@ -171,3 +171,8 @@ def test_graph_replayed_decode_matches_eager(selector_cls):
     assert int(cache._len32) == 400 + 1 + 2 + steps  # capture itself executes nothing
     with pytest.raises(NotImplementedError):
         OmniKVMulLM(SHAPE, _config("uniform", False)).to(DEV).capture_decode(cache, tok)
+    if offload:  # rows packed by host threads cannot be part of a graph
+        lm3 = fresh()
+        _, c3 = lm3.forward(ids, None, max_new_tokens=32, offload_mode="memcpy")
+        with pytest.raises(NotImplementedError):
+            lm3.capture_decode(c3, tok)
