@@ -208,7 +208,7 @@ __device__ __forceinline__ float quad_swap(float x) {
 }
 
 // ------------------------------------------------------------------ pass 2
-// grid (row blocks, batch), one wave per kv head; LDS: [window][rows_per_block] bit
+// grid (row blocks, batch), one wave per kv head; LDS: [window][rows_per_block + 1] bit
 // patterns of non-negative floats (their unsigned order is their numeric order).
 template <typename T, int NCB>
 __global__ __launch_bounds__(512) void window_score_mfma(WindowArgs a, int rows_per_block, int exp_decay,
@@ -223,7 +223,11 @@ __global__ __launch_bounds__(512) void window_score_mfma(WindowArgs a, int rows_
   const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
   const int r16 = lane & 15, j4 = lane >> 4;
 
-  for (int i = threadIdx.x; i < a.window * rows_per_block; i += blockDim.x) wmax[i] = 0u;
+  // rows one word apart per position: the 4 positions x 4 lane rows of one atomic instruction
+  // then fall into 16 different banks (a stride that is a multiple of 32 words puts the
+  // positions on one bank: 74% of the LDS cycles were conflicts)
+  const int wstride = rows_per_block + 1;
+  for (int i = threadIdx.x; i < a.window * wstride; i += blockDim.x) wmax[i] = 0u;
 
   uint4 qf[NCB][4];
   load_window_q<T, NCB>(a, b, g, r16, j4, qf);
@@ -262,7 +266,7 @@ __global__ __launch_bounds__(512) void window_score_mfma(WindowArgs a, int rows_
         if (a.group >= 4) p = fmaxf(p, quad_swap<0x4E>(p));
         if (a.group >= 8) p = fmaxf(p, __shfl_xor(p, 4));
         if (wcol[cb] >= 0 && row0 + i < end - begin)
-          atomicMax(&wmax[wcol[cb] * rows_per_block + row0 + i], __float_as_uint(p));
+          atomicMax(&wmax[wcol[cb] * wstride + row0 + i], __float_as_uint(p));
       }
     }
   };
@@ -289,7 +293,7 @@ __global__ __launch_bounds__(512) void window_score_mfma(WindowArgs a, int rows_
     // running sum halved before each addition (exp)
     float acc = __uint_as_float(wmax[r]);
     for (int w = 1; w < a.window; ++w) {
-      const float v = __uint_as_float(wmax[w * rows_per_block + r]);
+      const float v = __uint_as_float(wmax[w * wstride + r]);
       acc = exp_decay ? acc * 0.5f + v : acc + v;
     }
     scores[(int64_t)b * score_stride + begin + r] = acc;
@@ -329,10 +333,13 @@ static void launch_window(WindowArgs a, int batch, int exp_decay, float* scores,
   int rpb = (int)((per + 15) / 16 * 16);
   if (rpb < 64) rpb = 64;
   const int cap = (48 * 1024 / 4 / a.window) / 16 * 16;
-  if (rpb > cap) rpb = cap;
+  if (rpb > cap) {  // several rounds of one block per CU: equal ones
+    const int64_t rounds = (per + cap - 1) / cap;
+    rpb = (int)(((per + rounds - 1) / rounds + 15) / 16 * 16);
+  }
   dim3 grid((a.max_score_len + rpb - 1) / rpb, batch);
   hipLaunchKernelGGL((window_score_mfma<T, NCB>), grid, dim3(64 * a.hkv),
-                     (size_t)a.window * rpb * sizeof(uint32_t), stream, a, rpb, exp_decay, scores,
+                     (size_t)a.window * (rpb + 1) * sizeof(uint32_t), stream, a, rpb, exp_decay, scores,
                      score_stride);
 }
 
