@@ -93,6 +93,7 @@ int carve_attn_workspace(void* ws, size_t ws_bytes, int batch, int hq, int hkv, 
   memset(out, 0, sizeof(*out));
   out->split_rows = C;
   out->max_splits = S;
+  out->logit_heads = hq;
   if (with_v) {
     out->part_o = (float*)p;
     p += align_up((size_t)batch * hq * S * d * sizeof(float), 256);

@@ -249,9 +249,10 @@ __global__ __launch_bounds__(256) void score_finish(RowList rows, int hq, AttnWo
   const bool soft = normalise == OKV_NORM_SOFTMAX;
   const float init = is_max ? -INFINITY : 0.f;
   float acc[4] = {init, init, init, init};
-  const float* lg = w.logits + (int64_t)b * hq * w.logits_stride + t0;
+  const int nh = w.logit_heads;  // Hq, or Hkv when the split pass has folded each group already
+  const float* lg = w.logits + (int64_t)b * nh * w.logits_stride + t0;
 #pragma unroll 8
-  for (int h = 0; h < hq; ++h) {
+  for (int h = 0; h < nh; ++h) {
     const float4 v4 = *reinterpret_cast<const float4*>(lg + (int64_t)h * w.logits_stride);
     float v[4] = {v4.x, v4.y, v4.z, v4.w};
     const float lse = soft ? w.score_lse[b * hq + h] : 0.f;
@@ -309,9 +310,15 @@ static int launch_typed(const void* q, const RowList& rows, const okv_kv_layout_
     OKV_HIP_CHECK(hipGetLastError());
     return OKV_OK;
   }
+  AttnWorkspace wm = w;  // what the matrix-core kernel may do on top: fold the group for raw scores
+  if (want_scores && normalise == OKV_NORM_RAW && G > 1) {
+    wm.group_reduce = head_reduce == OKV_REDUCE_MAX ? 1 : 2;
+    wm.logit_heads = hkv;
+  }
+  const AttnWorkspace* used = &w;
   if (g_attn_variant != 1 &&
-      launch_stage1_mfma(lay->dtype, q, rows, hq, hkv, batch, scale, w, with_v, want_scores, stream)) {
-    // 16-bit K/V: stage 1 ran on the matrix-core kernel
+      launch_stage1_mfma(lay->dtype, q, rows, hq, hkv, batch, scale, wm, with_v, want_scores, stream)) {
+    used = &wm;  // 16-bit K/V: stage 1 ran on the matrix-core kernel
   } else
   switch (G) {
     case 1: launch_stage1<T, 1>(q, rows, hq, hkv, batch, scale, w, with_v, want_scores, stream); break;
@@ -322,11 +329,11 @@ static int launch_typed(const void* q, const RowList& rows, const okv_kv_layout_
   }
   const bool need_score_lse = want_scores && normalise == OKV_NORM_SOFTMAX;
   if (!g_skip_merge && (with_v || need_score_lse))
-    hipLaunchKernelGGL((attn_merge<T>), dim3(hq, batch), dim3(256), 0, stream, rows, hq, w,
+    hipLaunchKernelGGL((attn_merge<T>), dim3(hq, batch), dim3(256), 0, stream, rows, hq, *used,
                        (T*)out, (int)with_v, (int)need_score_lse);
   if (want_scores && rows.max_score_len > 0)
     hipLaunchKernelGGL(score_finish, dim3((rows.max_score_len + 1023) / 1024, batch), dim3(256), 0,
-                       stream, rows, hq, w, head_reduce, normalise, scores, score_stride);
+                       stream, rows, hq, *used, head_reduce, normalise, scores, score_stride);
   OKV_HIP_CHECK(hipGetLastError());
   return OKV_OK;
 }

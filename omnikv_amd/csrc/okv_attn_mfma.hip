@@ -222,9 +222,22 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
     for (int s = 0; s < 4; ++s) S = mfma16((const T*)nullptr, kf[s], qf[s], S);
     const int row0 = tbase + 4 * j4;
     const bool partial = tbase + 16 > end;  // wave-uniform
-    if (scored && r16 < G)  // staged in LDS, flushed after the loop: no global store in the loop
-      *reinterpret_cast<float4*>(slog + r16 * w.split_rows + (row0 - begin)) =
-          make_float4(S[0] * scale, S[1] * scale, S[2] * scale, S[3] * scale);
+    if (scored) {  // staged in LDS, flushed after the loop: no global store in the loop
+      float v[4] = {S[0] * scale, S[1] * scale, S[2] * scale, S[3] * scale};
+      if (w.group_reduce) {  // raw scores: fold the G q heads (lanes 0..G-1 of the lane row) here
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+          for (int o = 1; o < G; o <<= 1) {
+            const float x = __shfl_xor(v[i], o);
+            v[i] = w.group_reduce == 1 ? fmaxf(v[i], x) : v[i] + x;
+          }
+        }
+      }
+      if (r16 < (w.group_reduce ? 1 : G))
+        *reinterpret_cast<float4*>(slog + r16 * w.split_rows + (row0 - begin)) =
+            make_float4(v[0], v[1], v[2], v[3]);
+    }
     float s[4] = {S[0], S[1], S[2], S[3]};
     if (partial) {
 #pragma unroll
@@ -315,11 +328,12 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
   if (scored) {
     __syncthreads();
     const int quads = w.split_rows >> 2;
-    for (int o = threadIdx.x; o < G * quads; o += 256) {
+    const int nh = w.group_reduce ? 1 : G;  // logits rows this kv head contributes
+    for (int o = threadIdx.x; o < nh * quads; o += 256) {
       const int h = o / quads, r = begin + 4 * (o % quads);
       if (r >= end) continue;
       const float4 v = *reinterpret_cast<const float4*>(slog + h * w.split_rows + (r - begin));
-      float* lp = w.logits + (int64_t)(b * hq + g * G + h) * w.logits_stride + r;
+      float* lp = w.logits + (int64_t)(b * w.logit_heads + g * nh + h) * w.logits_stride + r;
       if (r + 3 < end) {
         *reinterpret_cast<float4*>(lp) = v;
       } else {

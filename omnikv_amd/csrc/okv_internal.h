@@ -135,6 +135,10 @@ struct AttnWorkspace {
   int32_t max_splits;
   int32_t split_rows;
   int64_t logits_stride;
+  // Raw scores need no per-head normaliser, so the split pass may fold the q heads of a kv
+  // head itself and leave one logits row per kv head: a quarter of the bytes at group 4.
+  int32_t group_reduce;  // 0 = one row per q head, 1 = max over the group, 2 = sum over the group
+  int32_t logit_heads;   // rows of `logits` per request: Hq, or Hkv when group_reduce
 };
 
 size_t attn_workspace_bytes(int batch, int hq, int hkv, int d, int max_main, int max_tail,
