@@ -49,12 +49,20 @@ def _stream_ptr(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
+_retired: list = []  # outgrown scratch buffers: captured graphs may still hold their addresses
+
+
 def _workspace(device, nbytes: int) -> torch.Tensor:
-    """One growing scratch buffer per (device, stream)."""
+    """One growing scratch buffer per (device, stream).  It at least doubles when it grows and
+    the buffer it replaces stays allocated (a HIP graph captured earlier keeps launching with
+    the old address), so what is held in total is bounded by twice the largest request."""
     key = (device.index if device.index is not None else torch.cuda.current_device(), _stream_ptr(device))
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        if ws is not None:
+            _retired.append(ws)
+        ws = torch.empty(max(nbytes, 1 << 20, 2 * ws.numel() if ws is not None else 0), dtype=torch.uint8,
+                         device=device)
         _workspaces[key] = ws
     return ws
 
