@@ -153,12 +153,12 @@ __global__ __launch_bounds__(256) void attn_stage1_generic(const T* __restrict__
 // thread folds its splits with a running max (all loads independent, one trip to
 // memory), then the 8 split lanes of a column meet in LDS.
 template <typename T>
-__global__ __launch_bounds__(256) void attn_merge(RowList rows, int hq, AttnWorkspace w,
-                                                  T* __restrict__ out, int with_v,
-                                                  int with_score_lse) {
+__device__ __forceinline__ void merge_body(const RowList& rows, int hq, const AttnWorkspace& w,
+                                           T* __restrict__ out, int with_v, int with_score_lse, int h,
+                                           int b) {
   __shared__ float4 snum[8][32];
   __shared__ float sm[8], sden[8], smA[8], sdenA[8];
-  const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+  const int tid = threadIdx.x;
   const int main_len = rl_main_len(rows, b);
   const int L = main_len + rl_tail_len(rows, b);
   const int A = rl_score_len(rows, b);
@@ -235,18 +235,62 @@ __global__ __launch_bounds__(256) void attn_merge(RowList rows, int hq, AttnWork
   }
 }
 
+template <typename T>
+__global__ __launch_bounds__(256) void attn_merge(RowList rows, int hq, AttnWorkspace w,
+                                                  T* __restrict__ out, int with_v,
+                                                  int with_score_lse) {
+  merge_body<T>(rows, hq, w, out, with_v, with_score_lse, blockIdx.x, blockIdx.y);
+}
+
 // ------------------------------------------------------------ score finish
-// grid (ceil(max_score/1024), batch), 256 threads, four consecutive tokens each.
-__global__ __launch_bounds__(256) void score_finish(RowList rows, int hq, AttnWorkspace w,
-                                                    int head_reduce, int normalise,
-                                                    float* __restrict__ scores,
-                                                    int64_t score_stride) {
-  const int b = blockIdx.y;
-  const int t0 = (blockIdx.x * 256 + threadIdx.x) * 4;
+// 256 threads, four consecutive tokens each, block `bx` of request `b`.  With own_lse the
+// block works out the per-head score normalisers itself from the splits' partial
+// log-sum-exps (a few KB from L2) instead of reading what a merge launch left, so that it
+// does not have to run after one.
+constexpr int kMaxFinishHeads = 256;
+__device__ __forceinline__ void finish_body(const RowList& rows, int hq, const AttnWorkspace& w,
+                                            int head_reduce, int normalise, float* __restrict__ scores,
+                                            int64_t score_stride, int bx, int b, bool own_lse) {
+  __shared__ float s_lse[kMaxFinishHeads];
+  const int t0 = (bx * 256 + threadIdx.x) * 4;
   const int A = rl_score_len(rows, b);
-  if (t0 >= A) return;
   const bool is_max = head_reduce == OKV_REDUCE_MAX;
   const bool soft = normalise == OKV_NORM_SOFTMAX;
+  if (soft && own_lse) {  // 8 threads per head, 32 heads per trip
+    const int nA = (A + w.split_rows - 1) / w.split_rows;
+    const int sub = threadIdx.x & 7;
+    for (int h0 = 0; h0 < hq; h0 += 32) {
+      const int h = h0 + (threadIdx.x >> 3);
+      float M = -INFINITY, d = 0.f;
+      if (h < hq) {
+        const float* pl = w.part_lse + (int64_t)(b * hq + h) * w.max_splits;
+        constexpr int U = 8;  // loads of a batch leave together
+        for (int s2 = sub; s2 < nA; s2 += 8 * U) {
+          float xs[U];
+#pragma unroll
+          for (int u = 0; u < U; ++u) xs[u] = s2 + 8 * u < nA ? pl[s2 + 8 * u] : -INFINITY;
+#pragma unroll
+          for (int u = 0; u < U; ++u) {
+            const float mn = fmaxf(M, xs[u]);
+            if (mn != -INFINITY) {
+              d = fmaf(d, exp2f(M - mn), exp2f(xs[u] - mn));
+              M = mn;
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int o = 1; o < 8; o <<= 1) {
+        const float M2 = __shfl_xor(M, o), d2 = __shfl_xor(d, o);
+        const float mn = fmaxf(M, M2);
+        if (mn != -INFINITY) d = d * exp2f(M - mn) + d2 * exp2f(M2 - mn);
+        M = mn;
+      }
+      if (h < hq && sub == 0) s_lse[h] = M + log2f(d);
+    }
+    __syncthreads();
+  }
+  if (t0 >= A) return;
   const float init = is_max ? -INFINITY : 0.f;
   float acc[4] = {init, init, init, init};
   const int nh = w.logit_heads;  // Hq, or Hkv when the split pass has folded each group already
@@ -255,7 +299,7 @@ __global__ __launch_bounds__(256) void score_finish(RowList rows, int hq, AttnWo
   for (int h = 0; h < nh; ++h) {
     const float4 v4 = *reinterpret_cast<const float4*>(lg + (int64_t)h * w.logits_stride);
     float v[4] = {v4.x, v4.y, v4.z, v4.w};
-    const float lse = soft ? w.score_lse[b * hq + h] : 0.f;
+    const float lse = soft ? (own_lse ? s_lse[h] : w.score_lse[b * hq + h]) : 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       float x = soft ? exp2f(v[i] * kLog2e - lse) : v[i];
@@ -270,6 +314,30 @@ __global__ __launch_bounds__(256) void score_finish(RowList rows, int hq, AttnWo
     for (int i = 0; i < 4; ++i)
       if (t0 + i < A) sp[i] = acc[i];
   }
+}
+
+// grid (ceil(max_score/1024), batch)
+__global__ __launch_bounds__(256) void score_finish(RowList rows, int hq, AttnWorkspace w,
+                                                    int head_reduce, int normalise,
+                                                    float* __restrict__ scores,
+                                                    int64_t score_stride) {
+  finish_body(rows, hq, w, head_reduce, normalise, scores, score_stride, blockIdx.x, blockIdx.y, false);
+}
+
+// Both in one launch: blocks [0, merge_blocks) fold the splits of one q head each, the rest
+// finish the scores (with their own normalisers: nothing here waits for another block).
+// grid (merge_blocks + ceil(max_score/1024), batch)
+template <typename T>
+__global__ __launch_bounds__(256) void merge_and_finish(RowList rows, int hq, AttnWorkspace w,
+                                                        T* __restrict__ out, int merge_blocks,
+                                                        int head_reduce, int normalise,
+                                                        float* __restrict__ scores,
+                                                        int64_t score_stride) {
+  if ((int)blockIdx.x < merge_blocks)
+    merge_body<T>(rows, hq, w, out, 1, 0, blockIdx.x, blockIdx.y);
+  else
+    finish_body(rows, hq, w, head_reduce, normalise, scores, score_stride, blockIdx.x - merge_blocks,
+                blockIdx.y, true);
 }
 
 // ----------------------------------------------------------------- launch
@@ -328,12 +396,20 @@ static int launch_typed(const void* q, const RowList& rows, const okv_kv_layout_
     default: set_error("GQA group %d not supported", G); return OKV_ERR_UNSUPPORTED;
   }
   const bool need_score_lse = want_scores && normalise == OKV_NORM_SOFTMAX;
-  if (!g_skip_merge && (with_v || need_score_lse))
-    hipLaunchKernelGGL((attn_merge<T>), dim3(hq, batch), dim3(256), 0, stream, rows, hq, *used,
-                       (T*)out, (int)with_v, (int)need_score_lse);
-  if (want_scores && rows.max_score_len > 0)
-    hipLaunchKernelGGL(score_finish, dim3((rows.max_score_len + 1023) / 1024, batch), dim3(256), 0,
-                       stream, rows, hq, *used, head_reduce, normalise, scores, score_stride);
+  const int finish_blocks = want_scores ? (rows.max_score_len + 1023) / 1024 : 0;
+  if (!g_skip_merge && finish_blocks > 0 && hq <= kMaxFinishHeads) {
+    // one launch: the merge of the outputs next to the finishing of the scores
+    hipLaunchKernelGGL((merge_and_finish<T>), dim3((with_v ? hq : 0) + finish_blocks, batch), dim3(256), 0,
+                       stream, rows, hq, *used, (T*)out, with_v ? hq : 0, head_reduce, normalise, scores,
+                       score_stride);
+  } else {
+    if (!g_skip_merge && (with_v || need_score_lse))
+      hipLaunchKernelGGL((attn_merge<T>), dim3(hq, batch), dim3(256), 0, stream, rows, hq, *used,
+                         (T*)out, (int)with_v, (int)need_score_lse);
+    if (finish_blocks > 0)
+      hipLaunchKernelGGL(score_finish, dim3(finish_blocks, batch), dim3(256), 0, stream, rows, hq, *used,
+                         head_reduce, normalise, scores, score_stride);
+  }
   OKV_HIP_CHECK(hipGetLastError());
   return OKV_OK;
 }
