@@ -29,7 +29,7 @@ import torch
 from . import ops
 from ._lib import check, lib
 
-__all__ = ["OmniKVMultiStageCache", "get_cache_cls", "layer_schedule"]
+__all__ = ["OmniKVMultiStageCache", "WOPackCache", "get_cache_cls", "get_idx_iou_score", "layer_schedule"]
 
 
 def layer_schedule(full_attn_layers, num_hidden_layers: int, num_wait_load_layers: int):

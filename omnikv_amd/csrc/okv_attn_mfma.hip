@@ -2,9 +2,10 @@
 // q.K^T contraction on the matrix cores.
 //
 // A wave owns 16-row tiles of one kv head.  q.K^T for the tile is four
-// v_mfma_f32_16x16x32 (K rows are the A operand straight from global memory: lane l
-// holds row l%16, elements 32s + 8(l/16) .. +8 of k-step s; the G q heads of the kv
-// head are the first G columns of the B operand, the rest zero).  The result leaves
+// v_mfma_f32_16x16x32 (K rows are the A operand: lane l holds row l%16, elements
+// 32s + 8(l/16) .. +8 of k-step s -- loaded in that layout by the gather modes, loaded as
+// whole streamed rows and turned into it through LDS by the streaming modes; the G q
+// heads of the kv head are the first G columns of the B operand, the rest zero).  The result leaves
 // lane l holding column (head) l%16 of tile rows 4(l/16) .. +4: the lanes of one
 // 16-lane row hold all heads of the same four rows, so each row of lanes keeps its
 // own online softmax, and the probabilities reach the P.V lanes by DPP row
