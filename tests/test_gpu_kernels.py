@@ -374,3 +374,37 @@ def test_group_sizes_one_two_eight(hq, hkv, dtype):
     ks = torch.cat([orc.gather_rows(k[:, :, :n], idx.cpu().to(torch.int64)), k[:, :, n:]], dim=2)
     vs = torch.cat([orc.gather_rows(v[:, :, :n], idx.cpu().to(torch.int64)), v[:, :, n:]], dim=2)
     assert (sp.cpu().float() - orc.gqa_attention(q.float(), ks.float(), vs.float())[:, :, 0]).abs().max() < tol
+
+
+def test_empty_requests_in_a_batch():
+    """A request of length zero next to ordinary ones: its attention output is defined as
+    zero, it gets no scores and selects nothing; the others are unaffected."""
+    lens = [0, 5, 300, 0, 1]
+    g = torch.Generator().manual_seed(31)
+    nmax = max(lens)
+    q = torch.randn((len(lens), 32, 1, 128), generator=g).to(torch.bfloat16)
+    k = torch.randn((len(lens), 8, nmax, 128), generator=g).to(torch.bfloat16)
+    v = torch.randn((len(lens), 8, nmax, 128), generator=g).to(torch.bfloat16)
+    sl = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    for sel in ("last", "softmax_sum_last"):
+        out, sc = ops.dense_attn(q.to(DEV), k.to(DEV), v.to(DEV), seq_len=nmax, seq_lens=sl, selector=sel,
+                                 score_len=nmax, score_lens=sl)
+        for b, n in enumerate(lens):
+            if n == 0:
+                assert float(out[b].float().abs().max()) == 0.0
+                continue
+            want = orc.gqa_attention(q[b:b + 1].float(), k[b:b + 1, :, :n].float(), v[b:b + 1, :, :n].float())[0, :, 0]
+            assert (out[b].cpu().float() - want).abs().max() < 2e-2
+            ws = orc.score_tokens(q[b:b + 1].float(), k[b:b + 1].float(), n, sel)[0]
+            assert _rel_err(sc[b:b + 1, :n].cpu(), ws[None]) < 1e-4
+    k_per = torch.tensor([0, 2, 20, 0, 1], dtype=torch.int32)
+    idx = torch.full((len(lens), 20), -1, dtype=torch.int32, device=DEV)
+    ops.topk(sc, 20, seq_lens=sl, k_per_seg=k_per.to(DEV), out=idx)
+    assert (idx[0] == -1).all() and (idx[3] == -1).all() and (idx[1, 2:] == -1).all()
+    sp = ops.sparse_attn(q.to(DEV), k.to(DEV), v.to(DEV), idx=idx, sel_len=20, sel_lens=k_per.to(DEV))
+    assert float(sp[0].float().abs().max()) == 0.0 and float(sp[3].float().abs().max()) == 0.0
+    for b in (1, 2, 4):
+        ii = idx[b, :int(k_per[b])].cpu().to(torch.int64)[None]
+        want = orc.gqa_attention(q[b:b + 1].float(), orc.gather_rows(k[b:b + 1], ii).float(),
+                                 orc.gather_rows(v[b:b + 1], ii).float())[0, :, 0]
+        assert (sp[b].cpu().float() - want).abs().max() < 2e-2
