@@ -40,9 +40,13 @@ static int num_compute_units() {
 // finish together, in one round when the split fits the row cap, else in the fewest
 // equal rounds.  The cap keeps the LDS staging of a scored split's logits small.
 static int choose_split_rows(int batch, int hq, int hkv, int total_rows, bool with_v,
-                             bool with_logits) {
+                             bool with_logits, bool gather) {
   if (g_split_rows_override > 0) return g_split_rows_override;
-  const int64_t capacity = (int64_t)num_compute_units() * (with_v ? 3 : 6);
+  // workgroups the chip runs side by side: the gather pass (selected rows through an index) is
+  // a chain of latencies and does best in exactly one round of two per CU -- measured: 192
+  // rows at 8781 selected rows, 512 at 30150; the streaming passes in 1.5 rounds of three
+  // (a batch is sized by its longest request, so ragged ones fill less than that: three there too)
+  const int64_t capacity = (int64_t)num_compute_units() * (gather && batch <= 1 ? 2 : with_v ? 3 : 6);
   // a scored split stages G*rows fp32 logits in LDS: keep that within 32 KB
   const int group = hkv > 0 && hq >= hkv ? hq / hkv : 1;
   const int64_t cap_rows = with_logits ? (8192 / group) / 64 * 64 : 4096;
@@ -50,9 +54,8 @@ static int choose_split_rows(int batch, int hq, int hkv, int total_rows, bool wi
   for (int64_t rounds = 1;; ++rounds) {
     int64_t rows = (work + rounds * capacity - 1) / (rounds * capacity);
     rows = (rows + 63) / 64 * 64;
-    if (rounds == 1 && with_v && rows <= 128) {
-      // a few thousand rows (sparse layers): the pass is a latency chain, and fewer, fatter
-      // workgroups (three tiles per wave, a third fewer partials to merge) finish sooner
+    if (rounds == 1 && with_v && !(gather && batch <= 1) && rows <= 128) {
+      // a short dense pass is a latency chain too: fewer, fatter workgroups
       rows = (work + capacity * 2 / 3 - 1) / (capacity * 2 / 3);
       rows = (rows + 63) / 64 * 64;
     }
@@ -62,9 +65,9 @@ static int choose_split_rows(int batch, int hq, int hkv, int total_rows, bool wi
 
 size_t attn_workspace_bytes(int batch, int hq, int hkv, int d, int max_main, int max_tail,
                             int max_score, bool with_v, bool with_logits, int* split_rows,
-                            int* max_splits) {
+                            int* max_splits, bool gather) {
   int L = max_main + max_tail;
-  int C = choose_split_rows(batch, hq, hkv, L, with_v, with_logits);
+  int C = choose_split_rows(batch, hq, hkv, L, with_v, with_logits, gather);
   int S = (L + C - 1) / C + (max_score > 0 ? 1 : 0);
   if (S < 1) S = 1;
   if (split_rows) *split_rows = C;
@@ -82,10 +85,10 @@ size_t attn_workspace_bytes(int batch, int hq, int hkv, int d, int max_main, int
 
 int carve_attn_workspace(void* ws, size_t ws_bytes, int batch, int hq, int hkv, int d,
                          int max_main, int max_tail, int max_score, bool with_v,
-                         bool with_logits, AttnWorkspace* out) {
+                         bool with_logits, AttnWorkspace* out, bool gather) {
   int C = 0, S = 0;
   size_t need = attn_workspace_bytes(batch, hq, hkv, d, max_main, max_tail, max_score, with_v,
-                                     with_logits, &C, &S);
+                                     with_logits, &C, &S, gather);
   OKV_REQUIRE(ws != nullptr, OKV_ERR_INVALID, "workspace pointer is NULL");
   OKV_REQUIRE(ws_bytes >= need, OKV_ERR_WORKSPACE, "workspace too small: have %zu, need %zu",
               ws_bytes, need);
@@ -177,7 +180,7 @@ int okv_workspace_bytes(int op, const okv_shape_t* s, size_t* out_bytes) {
     case OKV_OP_SPARSE_ATTN:
       *out_bytes = okv::attn_workspace_bytes(s->batch, s->num_q_heads, s->num_kv_heads, s->head_dim,
                                              s->max_seq_len, s->max_tail_len, 0, true, false,
-                                             nullptr, nullptr);
+                                             nullptr, nullptr, true);
       return OKV_OK;
     case OKV_OP_TOPK:
       *out_bytes = okv::topk_mb_workspace_bytes(s->batch, s->max_seq_len);

@@ -559,7 +559,7 @@ int okv_sparse_attn(const void* q, const void* k_base, const void* v_base,
   }
   AttnWorkspace w;
   rc = carve_attn_workspace(ws, ws_bytes, batch, layout->num_q_heads, layout->num_kv_heads,
-                            layout->head_dim, max_sel_len, max_tail_len, 0, true, false, &w);
+                            layout->head_dim, max_sel_len, max_tail_len, 0, true, false, &w, true);
   if (rc) return rc;
   RowList r;
   fill_main(&r, k_base, v_base, layout);

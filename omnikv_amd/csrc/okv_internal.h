@@ -143,10 +143,10 @@ struct AttnWorkspace {
 
 size_t attn_workspace_bytes(int batch, int hq, int hkv, int d, int max_main, int max_tail,
                             int max_score, bool with_v, bool with_logits,
-                            int* split_rows, int* max_splits);
+                            int* split_rows, int* max_splits, bool gather = false);
 int carve_attn_workspace(void* ws, size_t ws_bytes, int batch, int hq, int hkv, int d,
                          int max_main, int max_tail, int max_score, bool with_v,
-                         bool with_logits, AttnWorkspace* out);
+                         bool with_logits, AttnWorkspace* out, bool gather = false);
 
 extern int g_split_rows_override;  // 0 = automatic
 
