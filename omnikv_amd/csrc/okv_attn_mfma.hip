@@ -144,8 +144,9 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
         // pages of 16k rows: the whole tile lies in one page, looked up once through the scalar unit
         const int tb = __builtin_amdgcn_readfirstlane(tbase);
         tr.tok[x] = rows.page_table[(int64_t)b * rows.page_table_stride + (tb >> rows.page_shift)];
-      } else if (MODE == 1) {  // branch-free: main_len >= 1 is guaranteed by the launcher
-        const int ri = r < main_len ? r : main_len - 1;
+      } else if (MODE == 1) {  // branch-free: the index holds at least one entry per request
+        int ri = r < main_len ? r : main_len - 1;
+        ri = ri < 0 ? 0 : ri;  // a request with tail rows only
         const int t = idx_row[ri];
         tr.tok[x] = r < main_len ? t : r - main_len;
       } else if (r >= main_len) {
@@ -407,7 +408,7 @@ static void launch_g(const void* q, const RowList& rows, int hq, int hkv, int ba
   const bool no_tail = rows.max_tail_len == 0 && !rows.tail_lens;
   int mode = 2;
   if (!rows.idx && !rows.page_table && no_tail) mode = 0;
-  else if (rows.idx && !rows.page_table && !rows.main_lens && rows.max_main_len >= 1) mode = 1;
+  else if (rows.idx && !rows.page_table && rows.max_main_len >= 1) mode = 1;
   else if (rows.page_table && !rows.idx && no_tail && rows.page_shift >= 4) mode = 3;
 #define OKV_MODES(WV, LG)                                                                  \
   do {                                                                                     \

@@ -26,7 +26,7 @@ def main():
     ap.add_argument("--op", required=True,
                     choices=["dense", "fused", "score", "topk", "sparse", "sparse_packed", "gather", "copy",
                              "offload_memcpy", "offload_zero_copy", "h2d", "window", "window_loop",
-                             "paged_dense", "paged_fused", "paged_score", "paged_topk", "paged_sparse"])
+                             "paged_dense", "paged_fused", "paged_score", "paged_topk", "paged_sparse", "paged_sparse_slots"])
     ap.add_argument("--batch", type=int, default=16, help="requests of the paged_* ops (ragged lengths 8192..32768)")
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--pages-in-order", action="store_true", help="paged_* ops: identity page table instead of shuffled")
@@ -206,6 +206,8 @@ def paged(args, dev):
     idx = torch.zeros((args.batch, kmax), dtype=torch.int32, device=dev)
     ops.topk(scores, kmax, seq_lens=lens_d, k_per_seg=k_per_d, out=idx)
 
+    slots = pools[0].slot_index(idx) if args.op == "paged_sparse_slots" else None
+
     def call(i):
         l = i % nl
         if args.op == "paged_dense":
@@ -217,13 +219,15 @@ def paged(args, dev):
             return score_(qs[l], pools[l], score_len=nmax, selector=args.selector, score_lens=lens_d)
         if args.op == "paged_topk":
             return ops.topk(scores, kmax, seq_lens=lens_d, k_per_seg=k_per_d, out=idx)
+        if args.op == "paged_sparse_slots":
+            return ops.sparse_attn(qs[l], pools[l], slots=slots, sel_len=kmax, sel_lens=k_per_d)
         return sparse_(qs[l], pools[l], idx=idx, sel_len=kmax, sel_lens=k_per_d)
 
     tokens, sel = int(lens.sum()), int(k_per.sum())
     row = HKV * D * es
     algo = {"paged_dense": 2.0 * tokens * row, "paged_fused": 2.0 * tokens * row + 4.0 * tokens,
             "paged_score": 1.0 * tokens * row + 4.0 * tokens, "paged_topk": 4.0 * tokens + 4.0 * sel,
-            "paged_sparse": 2.0 * sel * row + 4.0 * sel}[args.op]
+            "paged_sparse": 2.0 * sel * row + 4.0 * sel, "paged_sparse_slots": 2.0 * sel * row + 4.0 * sel}[args.op]
     for i in range(args.warmup):
         call(i)
     torch.cuda.synchronize()

@@ -41,6 +41,19 @@ class PagedKV:
     page_table: torch.Tensor
     page_size: int
 
+    def slot_index(self, idx: torch.Tensor) -> torch.Tensor:
+        """Token positions (bsz, k) int32 -> rows of the pool seen as one flat array of token
+        slots: page_table[b, t // page_size] * page_size + t % page_size.  Composed once per
+        selection (the reference's serving stack keeps exactly such a table per request,
+        req_to_imp_token_indexs, common/req_manager.py:12-17), every sparse layer of the
+        group then reads its rows with one lookup instead of two.  Padding entries (< 0)
+        stay padding."""
+        if self.pool_k.stride(0) != self.page_size * self.pool_k.stride(1):
+            raise ValueError("the pool's pages must lie back to back")
+        t = idx.clamp(min=0).to(torch.int64)
+        slots = self.page_table.gather(1, t // self.page_size).to(torch.int64) * self.page_size + t % self.page_size
+        return torch.where(idx < 0, idx, slots.to(torch.int32))
+
 
 _workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
 
@@ -239,7 +252,8 @@ def dense_attn(q, k, v=None, seq_len: Optional[int] = None, seq_lens: Optional[t
 def sparse_attn(q, k, v=None, idx: Optional[torch.Tensor] = None, sel_len: Optional[int] = None,
                 sel_lens: Optional[torch.Tensor] = None, tail_k: Optional[torch.Tensor] = None,
                 tail_v: Optional[torch.Tensor] = None, tail_len: Optional[int] = None,
-                tail_lens: Optional[torch.Tensor] = None, scale: Optional[float] = None) -> torch.Tensor:
+                tail_lens: Optional[torch.Tensor] = None, scale: Optional[float] = None,
+                slots: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention over rows idx of K/V followed by the tail rows; okv_sparse_attn.
 
     idx (bsz, k) int32 ascending, or None for rows [0, sel_len).  tail_k / tail_v
@@ -247,7 +261,16 @@ def sparse_attn(q, k, v=None, idx: Optional[torch.Tensor] = None, sel_len: Optio
     q = _q3(q)
     _require_gpu(q, "q")
     hq, d = q.shape[1], q.shape[2]
-    lay, kp, vp, batch, n = _layout(k, v, hq)
+    if slots is not None:
+        # rows of a paged pool addressed as token slots (PagedKV.slot_index): no page table
+        if not isinstance(k, PagedKV) or idx is not None:
+            raise ValueError("slots go with a PagedKV and replace idx")
+        pool_k, pool_v = k.pool_k, k.pool_v
+        lay = KVLayout(_DTYPES[pool_k.dtype], hq, pool_k.shape[2], pool_k.shape[3], pool_k.stride(1),
+                       pool_k.stride(2), 0, None, 0, 0, 0)
+        kp, vp, batch, n, idx = pool_k.data_ptr(), pool_v.data_ptr(), slots.shape[0], None, slots
+    else:
+        lay, kp, vp, batch, n = _layout(k, v, hq)
     ip, istride = None, 0
     if idx is not None:
         if idx.dtype != torch.int32 or idx.dim() != 2 or idx.stride(1) != 1 or not idx.is_cuda:

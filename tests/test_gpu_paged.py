@@ -67,6 +67,14 @@ def test_paged_ragged_batch(page_size, dtype):
             want_sp = orc.gqa_attention(qn[b:b + 1].float(), orc.gather_rows(ks[b], want_idx).float(),
                                         orc.gather_rows(vs[b], want_idx).float())[0, :, 0]
             assert (sparse[b].cpu().float() - want_sp).abs().max() < tol
+        # the same rows through token slots composed once (one lookup per row instead of two)
+        slots = kv.slot_index(idx)
+        assert slots.dtype == torch.int32 and ((slots < 0) == (idx < 0)).all()
+        b0, k0 = 2, int(k_per[2])
+        t = idx[b0, :k0].cpu().long()
+        assert torch.equal(slots[b0, :k0].cpu().long(), table[b0, t // page_size].long() * page_size + t % page_size)
+        via_slots = ops.sparse_attn(qn.to(DEV), kv, slots=slots, sel_len=int(k_per.max()), sel_lens=k_per.to(DEV))
+        assert torch.equal(via_slots, sparse)  # identical rows in identical order: bit-identical output
     # LightLLM's own score: unscaled q.k, max over heads (rank-equivalent to `last`)
     raw = ops.score(q.to(DEV), kv, score_len=nmax, selector="last", scale=1.0, score_lens=lens_d)
     for b in (0, 5):
