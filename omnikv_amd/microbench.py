@@ -41,8 +41,9 @@ def main():
     ap.add_argument("--reps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--selector", default="softmax_sum_last")
-    ap.add_argument("--layout", default="hf", choices=["token_major", "hf"],
-                    help="hf = (1, Hkv, N, D) as the reference stores it; token_major = (1, N, Hkv, D)")
+    ap.add_argument("--layout", default="hf", choices=["token_major", "hf", "interleaved"],
+                    help="hf = (1, Hkv, N, D) as the reference stores it; token_major = (1, N, Hkv, D); "
+                         "interleaved = (1, Hkv, N, 2, D), K and V rows of a token side by side (times like hf)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32"])
     ap.add_argument("--split-rows", type=int, default=0)
     ap.add_argument("--attn-variant", type=int, default=0)
@@ -60,9 +61,13 @@ def main():
     gen = torch.Generator(device=dev).manual_seed(7)
     ks, vs, qs = [], [], []
     for _ in range(nl):
-        shape = (1, n + tail, HKV, D) if args.layout == "token_major" else (1, HKV, n + tail, D)
-        kb = torch.empty(shape, dtype=dtype, device=dev).normal_(generator=gen)
-        vb = torch.empty(shape, dtype=dtype, device=dev).normal_(generator=gen)
+        if args.layout == "interleaved":  # (1, Hkv, N, 2, D): a token's K and V rows of a head side by side
+            kvb = torch.empty((1, HKV, n + tail, 2, D), dtype=dtype, device=dev).normal_(generator=gen)
+            kb, vb = kvb[:, :, :, 0], kvb[:, :, :, 1]
+        else:
+            shape = (1, n + tail, HKV, D) if args.layout == "token_major" else (1, HKV, n + tail, D)
+            kb = torch.empty(shape, dtype=dtype, device=dev).normal_(generator=gen)
+            vb = torch.empty(shape, dtype=dtype, device=dev).normal_(generator=gen)
         if args.layout == "token_major":
             kb, vb = kb.permute(0, 2, 1, 3), vb.permute(0, 2, 1, 3)
         ks.append(kb)
