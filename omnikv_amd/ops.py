@@ -130,6 +130,11 @@ def _q3(q: torch.Tensor) -> torch.Tensor:
     return q.contiguous()
 
 
+def _same_dtype(q: torch.Tensor, lay) -> None:
+    if _DTYPES.get(q.dtype) != lay.dtype:
+        raise ValueError("q and K/V must have the same dtype (float32, bfloat16 or float16)")
+
+
 def _lens(t: Optional[torch.Tensor], batch: int, name: str) -> int:
     if t is None:
         return 0
@@ -145,6 +150,7 @@ def score(q, k, score_len: Optional[int] = None, selector: str = "last", scale: 
     _require_gpu(q, "q")
     hq, d = q.shape[1], q.shape[2]
     lay, kp, _, batch, n = _layout(k, None, hq)
+    _same_dtype(q, lay)
     if score_len is None:
         if n is None:
             raise ValueError("score_len is required with a paged pool")
@@ -181,6 +187,7 @@ def score_window(q, k, score_len: Optional[int] = None, selector: str = "uniform
         raise ValueError("q must be (bsz, Hq, W, D) with contiguous D")
     hq, w, d = q.shape[1], q.shape[2], q.shape[3]
     lay, kp, _, batch, n = _layout(k, None, hq)
+    _same_dtype(q, lay)
     if score_len is None:
         score_len = n
     if out is None:
@@ -224,6 +231,7 @@ def dense_attn(q, k, v=None, seq_len: Optional[int] = None, seq_lens: Optional[t
     _require_gpu(q, "q")
     hq, d = q.shape[1], q.shape[2]
     lay, kp, vp, batch, n = _layout(k, v, hq)
+    _same_dtype(q, lay)
     if seq_len is None:
         if n is None:
             raise ValueError("seq_len is required with a paged pool")
@@ -271,6 +279,7 @@ def sparse_attn(q, k, v=None, idx: Optional[torch.Tensor] = None, sel_len: Optio
         kp, vp, batch, n, idx = pool_k.data_ptr(), pool_v.data_ptr(), slots.shape[0], None, slots
     else:
         lay, kp, vp, batch, n = _layout(k, v, hq)
+    _same_dtype(q, lay)
     ip, istride = None, 0
     if idx is not None:
         if idx.dtype != torch.int32 or idx.dim() != 2 or idx.stride(1) != 1 or not idx.is_cuda:

@@ -408,3 +408,12 @@ def test_empty_requests_in_a_batch():
         want = orc.gqa_attention(q[b:b + 1].float(), orc.gather_rows(k[b:b + 1], ii).float(),
                                  orc.gather_rows(v[b:b + 1], ii).float())[0, :, 0]
         assert (sp[b].cpu().float() - want).abs().max() < 2e-2
+
+
+def test_mismatched_dtypes_are_refused():
+    q = torch.randn((1, 32, 1, 128), device=DEV)
+    k = torch.randn((1, 8, 64, 128), device=DEV).to(torch.bfloat16)
+    for call in (lambda: ops.score(q, k), lambda: ops.dense_attn(q, k, k), lambda: ops.sparse_attn(q, k, k),
+                 lambda: ops.score_window(q.expand(1, 32, 4, 128).contiguous(), k)):
+        with pytest.raises(ValueError, match="same dtype"):
+            call()
