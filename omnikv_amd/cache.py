@@ -130,6 +130,7 @@ class OmniKVMultiStageCache:
         self._copy_stream: Optional[torch.cuda.Stream] = None
         self._d2h_stream: Optional[torch.cuda.Stream] = None
         self._d2h_pending = False
+        self._d2h_staging: Optional[torch.Tensor] = None
         self._worker: Optional[threading.Thread] = None
         self._prefill_len: Optional[int] = None
         # static decode (enable_static_decode): lengths and write positions live on the device
@@ -245,8 +246,16 @@ class OmniKVMultiStageCache:
                 self._d2h_stream = torch.cuda.Stream(device=key_states.device)
             self._d2h_stream.wait_stream(cur)
             with torch.cuda.stream(self._d2h_stream):
-                host[:, 0].copy_(key_states[0].permute(1, 0, 2), non_blocking=True)
-                host[:, 1].copy_(value_states[0].permute(1, 0, 2), non_blocking=True)
+                # into the host layout on the GPU first (a strided device-to-host copy crawls at a
+                # few GB/s), then one contiguous copy at link speed; the staging buffer is reused
+                # layer after layer, in stream order
+                stg = self._d2h_staging
+                if stg is None or stg.shape != host.shape or stg.dtype != host.dtype:
+                    stg = torch.empty(host.shape, dtype=host.dtype, device=key_states.device)
+                    self._d2h_staging = stg
+                stg[:, 0].copy_(key_states[0].permute(1, 0, 2))
+                stg[:, 1].copy_(value_states[0].permute(1, 0, 2))
+                host.copy_(stg, non_blocking=True)
             key_states.record_stream(self._d2h_stream)
             value_states.record_stream(self._d2h_stream)
             self._d2h_pending = True
@@ -318,6 +327,7 @@ class OmniKVMultiStageCache:
         if self._d2h_pending:
             self._d2h_stream.synchronize()
             self._d2h_pending = False
+            self._d2h_staging = None  # half a gigabyte per layer at 128K: not kept past the prefill
 
     def _start_offload(self, idx32: torch.Tensor, layers: List[int]) -> None:
         if idx32.shape[0] != 1:
