@@ -417,3 +417,54 @@ def test_mismatched_dtypes_are_refused():
                  lambda: ops.score_window(q.expand(1, 32, 4, 128).contiguous(), k)):
         with pytest.raises(ValueError, match="same dtype"):
             call()
+
+
+def test_matrix_core_and_portable_kernels_agree_on_random_shapes():
+    """Seeded random geometries (lengths around tile / split boundaries, ragged batches, tails,
+    index lists, both layouts): the matrix-core kernels against the portable VALU kernels of
+    the same library, which share no load path, tile logic or split code with them."""
+    from omnikv_amd._lib import check, lib
+    rng = torch.Generator().manual_seed(2024)
+
+    def ri(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=rng))
+
+    try:
+        for case in range(24):
+            bsz = [1, 1, 2, 5][case % 4]
+            hkv = [8, 2, 4, 1][case % 4]
+            hq = hkv * [4, 8, 1, 2][(case // 4) % 4]
+            n = [1, 15, 16, 17, 63, 64, 65, 255, 256, 257, 1409, 2817, 5000][ri(0, 12)] + (ri(0, 3) if case % 3 else 0)
+            tail = [0, 1, 7, 40][ri(0, 3)]
+            lens = torch.tensor([ri(1, n) for _ in range(bsz)], dtype=torch.int32)
+            lens[ri(0, bsz - 1)] = n
+            dtype = [torch.bfloat16, torch.float16][case % 2]
+            q = torch.randn((bsz, hq, 1, 128), generator=rng).to(dtype).to(DEV)
+            k = torch.randn((bsz, hkv, n + tail, 128), generator=rng).to(dtype).to(DEV)
+            v = torch.randn((bsz, hkv, n + tail, 128), generator=rng).to(dtype).to(DEV)
+            if case % 5 == 0:
+                k, v = synth.token_major(k), synth.token_major(v)
+            ld = lens.to(DEV)
+            ksel = max(1, n // 7)
+            kper = torch.tensor([min(ksel, int(l)) for l in lens], dtype=torch.int32)
+            idx = torch.zeros((bsz, ksel), dtype=torch.int32)  # ascending per request, zero padded
+            for b in range(bsz):
+                idx[b, :int(kper[b])] = torch.randperm(int(lens[b]), generator=rng)[:int(kper[b])].sort().values
+            idx = idx.to(DEV)
+            res = {}
+            for variant in (0, 1):
+                check(lib().okv_set_option(b"attn_variant", variant))
+                o, sc = ops.dense_attn(q, k[:, :, :n], v[:, :, :n], seq_len=n, seq_lens=ld, selector="softmax_sum_last",
+                                       score_len=n, score_lens=ld)
+                raw = ops.score(q, k[:, :, :n], score_len=n, selector="last", score_lens=ld)
+                sp = ops.sparse_attn(q, k[:, :, :n], v[:, :, :n], idx=idx, sel_len=ksel, sel_lens=kper.to(DEV),
+                                     tail_k=k[:, :, n:] if tail else None, tail_v=v[:, :, n:] if tail else None)
+                res[variant] = (o.float(), sc, raw, sp.float())
+            for b in range(bsz):
+                lb = int(lens[b])
+                assert (res[0][0][b] - res[1][0][b]).abs().max() < 2e-2, (case, "dense", b)
+                assert _rel_err(res[0][1][b:b + 1, :lb].cpu(), res[1][1][b:b + 1, :lb].cpu()) < 1e-4, (case, "scores", b)
+                assert _rel_err(res[0][2][b:b + 1, :lb].cpu(), res[1][2][b:b + 1, :lb].cpu()) < 1e-4, (case, "raw", b)
+                assert (res[0][3][b] - res[1][3][b]).abs().max() < 2e-2, (case, "sparse", b)
+    finally:
+        check(lib().okv_set_option(b"attn_variant", 0))
