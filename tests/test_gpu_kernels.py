@@ -468,3 +468,39 @@ def test_matrix_core_and_portable_kernels_agree_on_random_shapes():
                 assert (res[0][3][b] - res[1][3][b]).abs().max() < 2e-2, (case, "sparse", b)
     finally:
         check(lib().okv_set_option(b"attn_variant", 0))
+
+
+def test_topk_random_lengths_and_distributions_bit_exact():
+    """Seeded random lengths on both sides of the single- / multi-workgroup switch, k from 1 to
+    n, smooth, quantised (many ties) and softmax-like scores, ragged batches: the indices must
+    equal the oracle's stable selection exactly."""
+    rng = torch.Generator().manual_seed(77)
+
+    def ri(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=rng))
+
+    for case in range(30):
+        bsz = [1, 1, 3][case % 3]
+        nmax = [ri(1, 300), ri(4000, 17000), ri(16384, 70000), ri(100000, 200000)][case % 4]
+        s = torch.randn((bsz, nmax), generator=rng)
+        kind = case % 5
+        if kind == 1:
+            s = torch.round(s * 4) / 4            # a few dozen distinct values: ties everywhere
+        elif kind == 2:
+            s = torch.softmax(s * 6, dim=-1)      # many tiny values, a few large
+        elif kind == 3:
+            s = s * 1e-30                         # near the subnormal range
+        elif kind == 4:
+            s[:, ::7] = 0.0
+            s[:, 1::13] = -0.0
+        lens = torch.tensor([ri(1, nmax) for _ in range(bsz)], dtype=torch.int32)
+        lens[ri(0, bsz - 1)] = nmax
+        kper = torch.tensor([ri(1, int(l)) if case % 2 else max(1, int(0.067 * int(l))) for l in lens], dtype=torch.int32)
+        kmax = int(kper.max())
+        out = torch.full((bsz, kmax), -1, dtype=torch.int32, device=DEV)
+        ops.topk(s.to(DEV), kmax, seq_lens=lens.to(DEV), k_per_seg=kper.to(DEV), out=out)
+        for b in range(bsz):
+            kb, lb = int(kper[b]), int(lens[b])
+            want = orc.select_topk_stable(s[b:b + 1, :lb], kb)[0]
+            assert torch.equal(out[b, :kb].cpu().to(torch.int64), want), (case, b, lb, kb)
+            assert (out[b, kb:] == -1).all()
