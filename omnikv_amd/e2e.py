@@ -32,7 +32,12 @@ def main():
     ap.add_argument("--offload-mode", default="zero_copy", choices=["zero_copy", "memcpy"])
     ap.add_argument("--full-attention", action="store_true", help="no selection: every layer attends to everything")
     ap.add_argument("--graph", action="store_true", help="replay the decode step from a HIP graph")
+    ap.add_argument("--trace", default=None, metavar="DESC",
+                    help="every layer reports its own selection each step (full attention, eager); writes "
+                         "debug_logs/selected_index_DESC.pt and prints the filter layers the run suggests")
     args = ap.parse_args()
+    if args.trace:
+        args.full_attention, args.graph = True, False
 
     dev = torch.device("cuda:0")
     shape = LlamaShape(num_hidden_layers=args.layers)
@@ -49,6 +54,11 @@ def main():
     torch.set_default_dtype(torch.float32)
     ids = torch.randint(0, shape.vocab_size, (1, args.ctx), generator=torch.Generator().manual_seed(1)).to(dev)
 
+    tracer = None
+    if args.trace:
+        from . import trace
+        tracer = trace.SelectedIndexTracer(desc=args.trace, num_selected_tokens=args.ratio)
+        trace.set_tracer(tracer)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     logits, cache = lm.forward(ids, None, max_new_tokens=args.steps + 16, offload_mode=args.offload_mode)
@@ -79,7 +89,14 @@ def main():
         dt = time.perf_counter() - t0
     if args.real_offload:
         cache._join_worker()
+    extra = {}
+    if tracer is not None:
+        mass, _ = tracer.matrices()
+        layers, quality = trace.suggest_filter_layers(mass, num_filters=len(args.select_layers.split(",")))
+        extra = {"trace_file": tracer.save_idx(), "suggested_select_layers": layers, "suggested_quality": quality,
+                 "configured_quality": trace.schedule_quality(mass, [int(i) for i in args.select_layers.split(",")])[0]}
     print(json.dumps({
+        **extra,
         "model": f"random-init Llama-3-8B shape, {args.layers} layers, bf16", "context": args.ctx,
         "decode_steps": args.steps, "select_layers": sel, "selected": int(args.ratio * args.ctx),
         "selector": args.selector, "real_offload": bool(args.real_offload and not args.full_attention),

@@ -16,6 +16,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from . import trace
 from .cache import OmniKVMultiStageCache, get_cache_cls
 from .config import OmniKVConfig
 from .selector import apply_rotary_pos_emb, select_from_query
@@ -140,6 +141,9 @@ class OmniKVMulLayer(nn.Module):
             if isinstance(num_selected_tokens, float):
                 num_selected_tokens = int(num_selected_tokens * consider_len)
             past_key_value.append(k, v, self.layer_idx)
+            if trace.idx_tracer is not None:
+                # every layer reports what it would select (modeling/offload_select_once.py:170-174)
+                trace.idx_tracer.observe(self.layer_idx, q, past_key_value.key_cache[self.layer_idx], consider_len)
             if self.layer_idx in self.do_select_layers:
                 if not self.config.get("dense_more", False):
                     raise ValueError("dense_more=False is not supported")
@@ -232,6 +236,8 @@ class OmniKVMulLM(nn.Module):
             position_ids = torch.arange(start, start + n, device=input_ids.device)[None].expand(input_ids.shape[0], -1)
         h = self.model(input_ids, position_ids, past_key_values)
         logits = self.lm_head(h[:, -1:]).float()
+        if trace.idx_tracer is not None and n == 1:
+            trace.idx_tracer.end_step(self.shape.num_hidden_layers)
         if static:
             past_key_values.advance_static()
         return logits, past_key_values
@@ -244,6 +250,8 @@ class OmniKVMulLM(nn.Module):
         by one -- a generation loop with no host work per token besides the replay."""
         if "last" not in self.config.get("selector_cls", "softmax_before_last"):
             raise NotImplementedError("the window selectors keep a host-side window; capture the `last` family")
+        if trace.idx_tracer is not None:
+            raise RuntimeError("selection tracing keeps per-step host state; trace an eager run")
         cache.enable_static_decode()
         token = first_token.clone().view(1, 1)
         stream = torch.cuda.Stream(device=token.device)

@@ -176,3 +176,65 @@ def test_graph_replayed_decode_matches_eager(selector_cls, offload):
         _, c3 = lm3.forward(ids, None, max_new_tokens=32, offload_mode="memcpy")
         with pytest.raises(NotImplementedError):
             lm3.capture_decode(c3, tok)
+
+
+def test_selection_tracing_compares_layers_and_leaves_decode_untouched(tmp_path):
+    """Every layer reports what it would select (the reference's SAVE_SELECTED_IDX runs):
+    the matrices are checked against the oracle's scores and stable top-k of the same
+    queries and keys, and a traced run generates what an untraced one does."""
+    from omnikv_amd import trace
+
+    cfg = _config("last", False)
+    lm = OmniKVMulLM(SHAPE, cfg).float().to(DEV)
+    lm.init_weights(seed=9, std=0.08)
+    n, steps, L = 400, 3, SHAPE.num_hidden_layers
+    ids = torch.randint(0, SHAPE.vocab_size, (1, n), generator=torch.Generator().manual_seed(4)).to(DEV)
+    plain, _ = lm.generate_greedy(ids, steps + 1)
+
+    seen = []  # (layer, q, K, consider_len) as the hook receives them
+
+    class Spy(trace.SelectedIndexTracer):
+        def observe(self, layer_idx, q, kview, consider_len):
+            seen.append((layer_idx, q.detach().cpu().clone(), kview[:, :, :consider_len].detach().cpu().clone()))
+            super().observe(layer_idx, q, kview, consider_len)
+
+    tr = Spy(desc="unit", num_selected_tokens=0.1, keep=5, save_dir=str(tmp_path))
+    assert trace.set_tracer(tr) is None
+    try:
+        traced, _ = lm.generate_greedy(ids, steps + 1)
+        with pytest.raises(RuntimeError):
+            lm.capture_decode(lm.new_cache(), plain[:, :1])
+    finally:
+        trace.set_tracer(None)
+    assert torch.equal(plain, traced)
+    assert tr.steps == steps and len(seen) == steps * L
+
+    k = int(0.1 * n)
+    mass = torch.zeros((L, L), dtype=torch.float64)
+    overlap = torch.zeros_like(mass)
+    for t in range(steps):
+        p, sel = [], []
+        for li, q, K in seen[t * L:(t + 1) * L]:
+            s = orc.score_tokens(q, K, n, "last")
+            p.append(torch.softmax(s[0].double(), -1))
+            sel.append(orc.select_topk_stable(s, k)[0])
+        for i in range(L):
+            for j in range(L):
+                mass[i, j] += p[j][sel[i]].sum()
+                overlap[i, j] += len(set(sel[i].tolist()) & set(sel[j].tolist())) / k
+    got_mass, got_overlap = tr.matrices()
+    assert (got_mass - mass / steps).abs().max() < 1e-4
+    assert (got_overlap - overlap / steps).abs().max() < 2.0 / k   # a near-tie may swap one index
+    assert torch.allclose(got_overlap.diagonal(), torch.ones(L, dtype=torch.float64))
+    # no other layer's choice keeps more of layer j's attention than layer j's own
+    assert (got_mass <= got_mass.diagonal()[None, :] + 1e-6).all()
+
+    path = tr.save_idx()
+    blob = trace.read_idx_tracer(path)
+    assert blob["steps"] == steps and torch.equal(blob["mass"], got_mass)
+    rec = blob["layers_idx"][0][2]
+    assert len(rec) == steps and rec[0]["idx"].shape == (1, 5) and rec[0]["prefill_len"] == n
+    assert (rec[0]["value"][0, :-1] >= rec[0]["value"][0, 1:]).all()
+    layers, quality = trace.suggest_filter_layers(got_mass, num_filters=2, num_wait_load_layers=1, max_dense_layers=5)
+    assert len(layers) == 2 and 0 < quality <= 1
+    assert quality == pytest.approx(trace.schedule_quality(got_mass, layers, 1)[0])

@@ -201,3 +201,37 @@ def test_rotary_matches_complex_rotation():
     z = torch.complex(x[..., : d // 2], x[..., d // 2:]) * torch.polar(torch.ones(d // 2, dtype=torch.float64), pos * inv)
     want = torch.cat([z.real, z.imag], dim=-1)
     assert torch.allclose(got, want, atol=1e-12)
+
+
+def test_filter_layer_suggestion_follows_the_cache_schedule():
+    """The tracer's schedule is the cache's own (which layers read which filter), and the
+    exhaustive search returns the planted optimum of a synthetic layer-agreement matrix."""
+    import itertools
+
+    from omnikv_amd import trace
+    from omnikv_amd.cache import layer_schedule
+
+    L = 12
+    for filters, wait in itertools.product([(2, 5, 9), (0, 6), (3,), (1, 2, 10)], [0, 1, 2]):
+        full = list(range(0, filters[0])) + list(filters) + [L]
+        want = {i: s[1] for i, s in layer_schedule(full, L, wait).items() if s[0]}
+        assert trace._schedule(filters, L, wait) == want
+    # layers fall into three groups that agree inside and not across; the best filters are the
+    # group heads, at the price of the layers before the first one staying dense
+    g = torch.tensor([0, 0, 1, 1, 1, 1, 2, 2, 2, 3, 3, 3])
+    mass = torch.where(g[:, None] == g[None, :], 0.9, 0.2).double()
+    layers, q = trace.suggest_filter_layers(mass, num_filters=3, num_wait_load_layers=1, max_dense_layers=8)
+    assert layers == [2, 6, 9] and q == pytest.approx(0.9)
+    assert trace.schedule_quality(mass, [2, 6, 9], 1) == (pytest.approx(0.9), 8)
+    assert trace.schedule_quality(mass, [1, 4, 8], 1)[0] < 0.9
+    with pytest.raises(ValueError):
+        trace.suggest_filter_layers(mass, num_filters=3, num_wait_load_layers=1, max_dense_layers=3)
+    # the recorder alone works without a GPU and round-trips through a file nothing is executed from
+    import tempfile
+    with tempfile.TemporaryDirectory() as d:
+        tr = trace.SelectedIndexTracer(desc="cpu", save_dir=d)
+        tr.append_spec_layer(torch.tensor([[3, 1]]), torch.tensor([[0.6, 0.4]]), 10, 7)
+        tr.append_out("text")
+        blob = trace.read_idx_tracer(tr.save_idx())
+        assert blob["out"] == ["text"] and blob["layers_idx"][0][7][0]["prefill_len"] == 10
+        assert torch.equal(blob["layers_idx"][0][7][0]["idx"], torch.tensor([[3, 1]]))
