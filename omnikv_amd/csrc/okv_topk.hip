@@ -17,7 +17,7 @@ static constexpr int kThreads = 1024;
 static constexpr int kWaves = kThreads / 64;
 static constexpr int kBins = 2048;
 static constexpr int kCandCap = 8192;  // candidate keys held in LDS (32 KB)
-static constexpr int kMultiBlockMinLen = 16384;  // below this one workgroup per request is faster
+static constexpr int kMultiBlockMinLen = 14336;  // below this one workgroup per request is faster
 
 __device__ __forceinline__ uint32_t score_key(float s) {
   uint32_t u = __float_as_uint(s);
@@ -317,7 +317,7 @@ extern "C" int okv_topk(const float* scores, int64_t score_stride, const int32_t
   int kk = max_k < max_seq_len ? max_k : max_seq_len;
   OKV_REQUIRE(idx_stride >= kk, OKV_ERR_INVALID, "idx_stride < min(max_k, max_seq_len)");
   if (max_seq_len == 0 || max_k == 0) return OKV_OK;
-  // long vectors: chunked multi-workgroup passes, if the caller brought the (zero-filled) workspace
+  // long vectors: chunked multi-workgroup passes, if the caller brought the workspace
   if (max_seq_len >= kMultiBlockMinLen && ws != nullptr &&
       ws_bytes >= topk_mb_workspace_bytes(batch, max_seq_len))
     return launch_topk_mb(scores, score_stride, seq_lens, max_seq_len, k_per_seg, max_k, batch,

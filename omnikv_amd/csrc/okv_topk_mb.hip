@@ -1,25 +1,34 @@
-// Top-k of long score vectors across many workgroups: a fill launch and four passes
-// over 4096-element chunks (one workgroup per chunk, the scores stay in L2).
+// Top-k of long score vectors across many workgroups, in three launches.  A request's scores
+// are cut into chunks of one or more 4096-key tiles, one workgroup of 1024 threads per chunk
+// (four keys per thread and tile: the work is chains of short dependent steps, and sixteen
+// waves per CU hide each other's latencies); the scores stay in L2 between the launches.
 //
-//   pass 0  zero the two shared histograms (a fill kernel, safe to capture in a graph)
-//   pass 1  histogram of the top 12 key bits            (LDS per chunk -> global atomics)
-//   pass 2  every workgroup scans that histogram, finds the bin of the k-th largest key,
-//           histograms the next 12 bits inside it, counts its keys above the bin
-//   pass 3  the same one level down; the low 8 bits inside the 24-bit prefix are
-//           histogrammed per chunk, privately
-//   pass 4  every workgroup sums the per-chunk low-bit histograms (all chunks: the exact
-//           threshold T and how many keys equal to T are taken; chunks before it: its
-//           output offset), then writes the indices of its chunk in order
+//   hist   every chunk histograms the top 12 bits of its keys in LDS and stores the histogram
+//          (16-bit counts) and its 256-bin summary in its own slot of the workspace
+//   cand   every workgroup sums the chunks' summaries, then the 16 bins inside the summary bin
+//          that holds the k-th largest key, which gives the bin B0 of that key; it copies the
+//          keys of its chunk that fall into B0 -- the candidates, a few percent of the chunk
+//          for smooth scores -- behind those of the chunks before it (their number is in the
+//          histograms it has just read), and counts its keys above B0
+//   write  every workgroup reads all candidates (kept in LDS when they fit), finds the exact
+//          threshold T among them over the remaining 20 bits in two 10-bit levels, counts what
+//          the chunks before its own hold above T and equal to T, and writes the selected
+//          indices of its chunk in order
 //
-// Grid-wide dependencies are kernel boundaries; no workgroup waits for another and
-// the workspace needs no preparation by the caller.
+// Nothing is accumulated across workgroups: no atomics on global memory, nothing to clear before
+// a call, no workgroup waits for another, and every count is an integer sum whose value does not
+// depend on the order of execution.
 #include "okv_internal.h"
 
 namespace okv {
 
-static constexpr int kChunk = 4096;
-static constexpr int kMbThreads = 256;
+static constexpr int kTile = 4096;         // keys per tile: 1024 threads x 4
+static constexpr int kMbThreads = 1024;
+static constexpr int kMbWaves = kMbThreads / 64;
 static constexpr int kBins12 = 4096;
+static constexpr int kMaxChunkTiles = 15;  // 61440 keys: a 16-bit count per bin cannot overflow
+static constexpr int kTargetChunks = 64;   // histograms every workgroup of `cand` sums
+static constexpr int kCandCache = 8192;    // candidates `write` keeps in LDS
 
 __device__ __forceinline__ uint32_t mb_key(float s) {
   uint32_t u = __float_as_uint(s);
@@ -28,119 +37,144 @@ __device__ __forceinline__ uint32_t mb_key(float s) {
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
-struct TopkMbState {  // per request, written by workgroup 0 of a pass for the later ones
-  uint32_t bin0, want1, bin1, want2;
+struct TopkMbState {  // per request, written by chunk 0 of `cand` for `write`
+  uint32_t bin0, want1, num_cand, pad;
 };
 
 struct TopkMbWs {
-  uint32_t* hist0;       // [batch][4096]
-  uint32_t* hist1;       // [batch][4096]
-  TopkMbState* state;    // [batch]
-  uint32_t* chunk_gt;    // [batch][max_chunks] keys above the 24-bit prefix, per chunk
-  uint16_t* chunk_low;   // [batch][max_chunks][256] low-byte histogram inside the prefix
+  uint16_t* hist0;      // [batch][max_chunks][4096]
+  uint16_t* coarse;     // [batch][max_chunks][256]  sums of 16 adjacent bins of hist0
+  uint32_t* cand;       // [batch][max_chunks * chunk_keys]  candidates, chunk after chunk, no gaps
+  uint32_t* cand_base;  // [batch][max_chunks]  where a chunk's candidates start
+  uint32_t* chunk_gt;   // [batch][max_chunks][16]  keys above the level-0 bin, per wave of the chunk's workgroup
+  TopkMbState* state;   // [batch]
   int max_chunks;
+  int chunk_tiles;
 };
 
+static void chunking(int max_seq_len, int* chunk_tiles, int* chunks) {
+  const int tiles = (max_seq_len + kTile - 1) / kTile;
+  int ct = (tiles + kTargetChunks - 1) / kTargetChunks;
+  if (ct < 1) ct = 1;
+  if (ct > kMaxChunkTiles) ct = kMaxChunkTiles;
+  *chunk_tiles = ct;
+  *chunks = (tiles + ct - 1) / ct;
+}
+
+static inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
+
 size_t topk_mb_workspace_bytes(int batch, int max_seq_len) {
-  const size_t chunks = (size_t)(max_seq_len + kChunk - 1) / kChunk;
+  int ct, chunks;
+  chunking(max_seq_len, &ct, &chunks);
   size_t b = 0;
-  b += (size_t)batch * kBins12 * 4 * 2;
-  b += (size_t)batch * sizeof(TopkMbState);
-  b += (size_t)batch * chunks * 4;
-  b += (size_t)batch * chunks * 256 * 2;
-  return b + 1024;
+  b += up256((size_t)batch * chunks * kBins12 * 2);
+  b += up256((size_t)batch * chunks * 256 * 2);
+  b += up256((size_t)batch * chunks * ct * kTile * 4);
+  b += up256((size_t)batch * chunks * 4);
+  b += up256((size_t)batch * chunks * kMbWaves * 4);
+  b += up256((size_t)batch * sizeof(TopkMbState));
+  return b + 256;
 }
 
 static TopkMbWs carve_topk(void* ws, int batch, int max_seq_len) {
   TopkMbWs w;
-  const size_t chunks = (size_t)(max_seq_len + kChunk - 1) / kChunk;
+  int ct, chunks;
+  chunking(max_seq_len, &ct, &chunks);
   char* p = (char*)(((uintptr_t)ws + 255) & ~(uintptr_t)255);
-  w.hist0 = (uint32_t*)p;
-  p += (size_t)batch * kBins12 * 4;
-  w.hist1 = (uint32_t*)p;
-  p += (size_t)batch * kBins12 * 4;
-  w.state = (TopkMbState*)p;
-  p += ((size_t)batch * sizeof(TopkMbState) + 255) & ~(size_t)255;
+  w.hist0 = (uint16_t*)p;
+  p += up256((size_t)batch * chunks * kBins12 * 2);
+  w.coarse = (uint16_t*)p;
+  p += up256((size_t)batch * chunks * 256 * 2);
+  w.cand = (uint32_t*)p;
+  p += up256((size_t)batch * chunks * ct * kTile * 4);
+  w.cand_base = (uint32_t*)p;
+  p += up256((size_t)batch * chunks * 4);
   w.chunk_gt = (uint32_t*)p;
-  p += ((size_t)batch * chunks * 4 + 255) & ~(size_t)255;
-  w.chunk_low = (uint16_t*)p;
-  w.max_chunks = (int)chunks;
+  p += up256((size_t)batch * chunks * kMbWaves * 4);
+  w.state = (TopkMbState*)p;
+  w.max_chunks = chunks;
+  w.chunk_tiles = ct;
   return w;
 }
 
-// 16 keys per thread of chunk `c`; element j of thread t is chunk element 4*(j/4*256 + t) + j%4
-// (coalesced float4s) or, with ORDERED, element 16*t + j (consecutive, for the final pass).
-template <bool ORDERED>
-__device__ __forceinline__ void load_chunk_keys(const float* __restrict__ s, int n, int c,
-                                                uint32_t (&key)[16], uint32_t& valid_mask) {
-  const int t = threadIdx.x;
-  const int base = c * kChunk;
-  const bool vec = (((uintptr_t)s) & 15) == 0;
+// Scores 4t .. 4t+3 of tile `tile` for thread t (one 16-byte load when aligned and in range).
+// Loading and key conversion are separate so that a kernel can issue the load first and wait
+// for it after its other memory round trips.
+__device__ __forceinline__ void load_tile_raw(const float* __restrict__ s, int n, int tile,
+                                              float (&x)[4], uint32_t& valid_mask) {
+  const int e = tile * kTile + 4 * threadIdx.x;
+  if ((((uintptr_t)s) & 15) == 0 && e + 3 < n) {
+    const float4 a = *reinterpret_cast<const float4*>(s + e);
+    x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w;
+    valid_mask = 0xfu;
+    return;
+  }
   valid_mask = 0;
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    const int e = ORDERED ? base + 16 * t + 4 * q : base + 4 * (q * kMbThreads + t);
-    float x[4];
-    if (vec && e + 3 < n) {
-      const float4 a = *reinterpret_cast<const float4*>(s + e);
-      x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w;
-      valid_mask |= 0xfu << (4 * q);
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        x[j] = (e + j < n) ? s[e + j] : 0.f;
-        if (e + j < n) valid_mask |= 1u << (4 * q + j);
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) key[4 * q + j] = mb_key(x[j]);
+  for (int j = 0; j < 4; ++j) {
+    x[j] = (e + j < n) ? s[e + j] : 0.f;
+    if (e + j < n) valid_mask |= 1u << j;
   }
 }
-
-// Every thread learns the bin (counted from the top) holding the `want`-th largest
-// element of a 4096-bin histogram in global memory, and the rank wanted inside it.
-__device__ void scan_hist12(const uint32_t* __restrict__ hist, uint32_t want, uint32_t* bin,
-                            uint32_t* want_in, uint32_t* sm /* >= 8 words of LDS */) {
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  // thread t owns bins 4095-16t .. 4080-16t (descending keys)
-  uint32_t h[16];
-  const uint4* hp = reinterpret_cast<const uint4*>(hist + (kBins12 - 16 * (t + 1)));
+__device__ __forceinline__ void keys_of(const float (&x)[4], uint32_t (&key)[4]) {
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    const uint4 v = hp[q];
+  for (int j = 0; j < 4; ++j) key[j] = mb_key(x[j]);
+}
+
+// Inclusive prefix sum over the 64 lanes of a wave.
+__device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const uint32_t u = __shfl_up(v, o);
+    if (lane >= o) v += u;
+  }
+  return v;
+}
+
+// Sum over the 64 lanes of a wave, in every lane.
+__device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
+// For ONE wave: the bin of an NB-bin histogram in LDS (16-byte aligned, complete) that holds the
+// `want`-th largest key, and the rank wanted inside it, in every lane.  Lane l takes bins
+// [NB - PER*(l+1), NB - PER*l): ascending lanes are descending keys.  A workgroup-wide scan
+// would cost three barriers of sixteen waves; this costs the callers one.
+template <int NB>
+__device__ __forceinline__ void wave_find_bin(const uint32_t* hist, uint32_t want, uint32_t& bin,
+                                              uint32_t& want_in) {
+  constexpr int PER = NB / 64;
+  const int lane = threadIdx.x & 63;
+  const int first = NB - PER * (lane + 1);
+  uint32_t h[PER];
+#pragma unroll
+  for (int q = 0; q < PER / 4; ++q) {
+    const uint4 v = reinterpret_cast<const uint4*>(hist + first)[q];
     h[4 * q] = v.x; h[4 * q + 1] = v.y; h[4 * q + 2] = v.z; h[4 * q + 3] = v.w;
   }
   uint32_t mine = 0;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) mine += h[i];
-  uint32_t inc = mine;
+  for (int i = 0; i < PER; ++i) mine += h[i];
+  const uint32_t inc = wave_scan(mine);
+  uint32_t run = inc - mine, fb = 0, fw = 1;
+  const bool found = run < want && want <= inc;  // at most one lane
+  if (found) {
 #pragma unroll
-  for (int o = 1; o < 64; o <<= 1) {
-    const uint32_t v = __shfl_up(inc, o);
-    if (lane >= o) inc += v;
-  }
-  __syncthreads();
-  if (lane == 63) sm[wave] = inc;
-  __syncthreads();
-  uint32_t off = 0;
-  for (int x = 0; x < wave; ++x) off += sm[x];
-  inc += off;
-  const uint32_t exc = inc - mine;
-  __syncthreads();
-  if (exc < want && want <= inc) {  // exactly one thread
-    uint32_t run = exc;
-#pragma unroll
-    for (int i = 15; i >= 0; --i) {  // h[15] is the thread's highest bin
+    for (int i = PER - 1; i >= 0; --i) {  // h[PER-1] is the lane's highest bin
       if (run < want && want <= run + h[i]) {
-        sm[4] = (uint32_t)(kBins12 - 16 * (t + 1) + i);
-        sm[5] = want - run;
+        fb = (uint32_t)(first + i);
+        fw = want - run;
       }
       run += h[i];
     }
   }
-  __syncthreads();
-  *bin = sm[4];
-  *want_in = sm[5];
+  const unsigned long long m = __ballot(found);
+  const int src = m ? __ffsll((long long)m) - 1 : 0;  // lane 0's defaults if the counts fell short
+  bin = __shfl(fb, src);
+  want_in = __shfl(fw, src);
 }
 
 __device__ __forceinline__ int req_len(const int32_t* seq_lens, int max_seq_len, int b) {
@@ -151,122 +185,174 @@ __device__ __forceinline__ int req_k(const int32_t* k_per_seg, int max_k, int b,
   return k < n ? k : n;
 }
 
-// LDS histogram of `bits` -> global atomics for the non-empty bins
-template <int NB>
-__device__ __forceinline__ void flush_hist(uint32_t* lh, uint32_t* __restrict__ gh) {
+__global__ __launch_bounds__(kMbThreads) void topk_mb_hist(const float* __restrict__ scores,
+                                                           int64_t score_stride,
+                                                           const int32_t* __restrict__ seq_lens,
+                                                           int max_seq_len,
+                                                           const int32_t* __restrict__ k_per_seg,
+                                                           int max_k, TopkMbWs w) {
+  __shared__ __attribute__((aligned(16))) uint32_t lh[kBins12];
+  const int c = blockIdx.x, b = blockIdx.y, t = threadIdx.x;
+  const int n = req_len(seq_lens, max_seq_len, b);
+  const int k = req_k(k_per_seg, max_k, b, n);
+  const int tile0 = c * w.chunk_tiles;
+  if ((int64_t)tile0 * kTile >= n || k <= 0 || k == n) return;
+  const float* s = scores + (int64_t)b * score_stride;
+  float x[4];
+  uint32_t valid;
+  load_tile_raw(s, n, tile0, x, valid);
+  reinterpret_cast<uint4*>(lh)[t] = make_uint4(0, 0, 0, 0);
   __syncthreads();
-  for (int i = threadIdx.x; i < NB; i += kMbThreads) {
-    const uint32_t v = lh[i];
-    if (v) atomicAdd(gh + i, v);
+  for (int i = 0;;) {
+    uint32_t key[4];
+    keys_of(x, key);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (valid >> j & 1) atomicAdd(&lh[key[j] >> 20], 1u);
+    if (++i >= w.chunk_tiles || (int64_t)(tile0 + i) * kTile >= n) break;
+    load_tile_raw(s, n, tile0 + i, x, valid);
+  }
+  __syncthreads();
+  // bins 4t .. 4t+3 as 16-bit counts, and the sum of 16 adjacent bins from four adjacent lanes
+  const uint4 a = reinterpret_cast<const uint4*>(lh)[t];
+  uint16_t* hp = w.hist0 + ((int64_t)b * w.max_chunks + c) * kBins12;
+  reinterpret_cast<uint2*>(hp)[t] = make_uint2(a.x | a.y << 16, a.z | a.w << 16);
+  uint32_t s16 = a.x + a.y + a.z + a.w;
+  s16 += __shfl_xor(s16, 1);
+  s16 += __shfl_xor(s16, 2);
+  if ((t & 3) == 0) w.coarse[((int64_t)b * w.max_chunks + c) * 256 + (t >> 2)] = (uint16_t)s16;
+}
+
+// the 16-bit halves of the four words of v, added to h[0..8)
+__device__ __forceinline__ void add_counts8(uint32_t* h, const uint4& v) {
+  const uint32_t e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (e[j] & 0xffffu) atomicAdd(&h[2 * j], e[j] & 0xffffu);
+    if (e[j] >> 16) atomicAdd(&h[2 * j + 1], e[j] >> 16);
   }
 }
 
-__global__ __launch_bounds__(kMbThreads) void topk_mb_pass0(uint4* __restrict__ p, int n16) {
-  const int i = blockIdx.x * kMbThreads + threadIdx.x;
-  if (i < n16) p[i] = make_uint4(0, 0, 0, 0);
-}
-
-__global__ __launch_bounds__(kMbThreads) void topk_mb_pass1(const float* __restrict__ scores,
-                                                            int64_t score_stride,
-                                                            const int32_t* __restrict__ seq_lens,
-                                                            int max_seq_len,
-                                                            const int32_t* __restrict__ k_per_seg,
-                                                            int max_k, TopkMbWs w) {
-  __shared__ uint32_t lh[kBins12];
-  const int c = blockIdx.x, b = blockIdx.y;
+__global__ __launch_bounds__(kMbThreads) void topk_mb_cand(const float* __restrict__ scores,
+                                                           int64_t score_stride,
+                                                           const int32_t* __restrict__ seq_lens,
+                                                           int max_seq_len,
+                                                           const int32_t* __restrict__ k_per_seg,
+                                                           int max_k, TopkMbWs w) {
+  __shared__ __attribute__((aligned(16))) uint32_t ch[256];  // the request's 256-bin summary
+  __shared__ uint32_t fh[16];   // its 16 fine bins inside the summary bin of the k-th key
+  __shared__ uint32_t fhb[16];  // the same over the chunks before this one
+  __shared__ uint32_t sm[4];
+  __shared__ uint32_t cnt;
+  const int c = blockIdx.x, b = blockIdx.y, t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int n = req_len(seq_lens, max_seq_len, b);
   const int k = req_k(k_per_seg, max_k, b, n);
-  if (c * kChunk >= n || k <= 0 || k == n) return;
-  for (int i = threadIdx.x; i < kBins12; i += kMbThreads) lh[i] = 0;
+  const int tile0 = c * w.chunk_tiles;
+  if ((int64_t)tile0 * kTile >= n || k <= 0 || k == n) return;
+  const int chunk_keys = w.chunk_tiles * kTile;
+  const int chunks = (n + chunk_keys - 1) / chunk_keys;
+  const float* s = scores + (int64_t)b * score_stride;
+  // the chunk's first tile is requested now and used after the two histogram round trips
+  float x[4];
+  uint32_t valid;
+  load_tile_raw(s, n, tile0, x, valid);
+  if (t < 256) ch[t] = 0;
+  if (t < 16) fh[t] = fhb[t] = 0;
+  if (t == 0) cnt = 0;
   __syncthreads();
-  uint32_t key[16], valid;
-  load_chunk_keys<false>(scores + (int64_t)b * score_stride, n, c, key, valid);
-#pragma unroll
-  for (int j = 0; j < 16; ++j)
-    if (valid >> j & 1) atomicAdd(&lh[key[j] >> 20], 1u);
-  flush_hist<kBins12>(lh, w.hist0 + (int64_t)b * kBins12);
-}
-
-__global__ __launch_bounds__(kMbThreads) void topk_mb_pass2(const float* __restrict__ scores,
-                                                            int64_t score_stride,
-                                                            const int32_t* __restrict__ seq_lens,
-                                                            int max_seq_len,
-                                                            const int32_t* __restrict__ k_per_seg,
-                                                            int max_k, TopkMbWs w) {
-  __shared__ uint32_t lh[kBins12];
-  __shared__ uint32_t sm[8];
-  const int c = blockIdx.x, b = blockIdx.y;
-  const int n = req_len(seq_lens, max_seq_len, b);
-  const int k = req_k(k_per_seg, max_k, b, n);
-  if (c * kChunk >= n || k <= 0 || k == n) return;
-  for (int i = threadIdx.x; i < kBins12; i += kMbThreads) lh[i] = 0;
+  // summaries of all chunks: chunks*32 16-byte pieces, piece l = chunk l/32, bins 8*(l%32) ..
+  {
+    const uint4* cp = reinterpret_cast<const uint4*>(w.coarse + (int64_t)b * w.max_chunks * 256);
+    const int pieces = chunks * 32;
+    for (int base = 0; base < pieces; base += 2 * kMbThreads) {
+      const int l0 = base + t, l1 = base + kMbThreads + t;
+      const uint4 v0 = l0 < pieces ? cp[l0] : make_uint4(0, 0, 0, 0);
+      const uint4 v1 = l1 < pieces ? cp[l1] : make_uint4(0, 0, 0, 0);
+      add_counts8(&ch[8 * (t & 31)], v0);  // kMbThreads is a multiple of 32: l % 32 == t % 32
+      add_counts8(&ch[8 * (t & 31)], v1);
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    uint32_t cb, wc;
+    wave_find_bin<256>(ch, (uint32_t)k, cb, wc);
+    if (lane == 0) {
+      sm[0] = cb;
+      sm[1] = wc;
+    }
+  }
+  __syncthreads();
+  const uint32_t cbin = sm[0], wantc = sm[1];
+  // the 16 fine bins inside it: two 16-byte pieces per chunk
+  {
+    const uint16_t* hp = w.hist0 + (int64_t)b * w.max_chunks * kBins12 + 16 * cbin;
+    for (int l = t; l < 2 * chunks; l += kMbThreads) {
+      const uint4 v = *reinterpret_cast<const uint4*>(hp + (int64_t)(l >> 1) * kBins12 + 8 * (l & 1));
+      add_counts8(&fh[8 * (l & 1)], v);
+      if ((l >> 1) < c) add_counts8(&fhb[8 * (l & 1)], v);
+    }
+  }
+  __syncthreads();
+  // the 16 bins from the top, one per lane (every wave does the same): lane j looks at bin 15-j
   uint32_t bin0, want1;
-  scan_hist12(w.hist0 + (int64_t)b * kBins12, (uint32_t)k, &bin0, &want1, sm);
-  if (c == 0 && threadIdx.x == 0) {
-    w.state[b].bin0 = bin0;
-    w.state[b].want1 = want1;
+  {
+    const uint32_t v = fh[15 - (lane & 15)];
+    uint32_t inc = v;
+#pragma unroll
+    for (int o = 1; o < 16; o <<= 1) {
+      const uint32_t u = __shfl_up(inc, o, 16);
+      if ((lane & 15) >= o) inc += u;
+    }
+    const bool found = lane < 16 && inc - v < wantc && wantc <= inc;
+    const unsigned long long m = __ballot(found);
+    const int src = m ? __ffsll((long long)m) - 1 : 0;
+    bin0 = 16 * cbin + 15 - src;
+    want1 = m ? wantc - __shfl(inc - v, src) : 1u;
   }
-  uint32_t key[16], valid;
-  load_chunk_keys<false>(scores + (int64_t)b * score_stride, n, c, key, valid);
+  // the candidates of a chunk are its keys in bin0, and every chunk's count of those is in the
+  // histograms just read: this chunk's candidates go right behind those of the chunks before it
+  const uint32_t base = fhb[bin0 & 15];
+  if (t == 0) {
+    w.cand_base[(int64_t)b * w.max_chunks + c] = base;
+    if (c == 0) {
+      w.state[b].bin0 = bin0;
+      w.state[b].want1 = want1;
+      w.state[b].num_cand = fh[bin0 & 15];
+    }
+  }
+  uint32_t* cand = w.cand + (int64_t)b * w.max_chunks * chunk_keys + base;
   uint32_t gt = 0;
+  for (int i = 0;;) {
+    uint32_t key[4];
+    keys_of(x, key);
+    uint32_t cmask = 0;
 #pragma unroll
-  for (int j = 0; j < 16; ++j) {
-    if (!(valid >> j & 1)) continue;
-    const uint32_t top = key[j] >> 20;
-    if (top > bin0) ++gt;
-    else if (top == bin0) atomicAdd(&lh[(key[j] >> 8) & 0xfffu], 1u);
+    for (int j = 0; j < 4; ++j) {
+      if (!(valid >> j & 1)) continue;
+      const uint32_t top = key[j] >> 20;
+      if (top > bin0) ++gt;
+      else if (top == bin0) cmask |= 1u << j;
+    }
+    // one LDS atomic per wave reserves room for the wave's candidates; their order is free
+    const uint32_t pc = __popc(cmask);
+    const uint32_t inc = wave_scan(pc);
+    const uint32_t wave_total = __shfl(inc, 63);
+    if (wave_total) {
+      uint32_t at = 0;
+      if (lane == 63) at = atomicAdd(&cnt, wave_total);
+      at = __shfl(at, 63) + inc - pc;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (cmask >> j & 1) cand[at++] = key[j];
+    }
+    if (++i >= w.chunk_tiles || (int64_t)(tile0 + i) * kTile >= n) break;
+    load_tile_raw(s, n, tile0 + i, x, valid);
   }
-  // keys of this chunk above the level-0 bin
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) gt += __shfl_xor(gt, o);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = gt;
-  __syncthreads();
-  if (threadIdx.x == 0) w.chunk_gt[(int64_t)b * w.max_chunks + c] = sm[0] + sm[1] + sm[2] + sm[3];
-  flush_hist<kBins12>(lh, w.hist1 + (int64_t)b * kBins12);
+  gt = wave_sum(gt);
+  if (lane == 0) w.chunk_gt[((int64_t)b * w.max_chunks + c) * kMbWaves + wave] = gt;
 }
 
-__global__ __launch_bounds__(kMbThreads) void topk_mb_pass3(const float* __restrict__ scores,
-                                                            int64_t score_stride,
-                                                            const int32_t* __restrict__ seq_lens,
-                                                            int max_seq_len,
-                                                            const int32_t* __restrict__ k_per_seg,
-                                                            int max_k, TopkMbWs w) {
-  __shared__ uint32_t low[256];
-  __shared__ uint32_t sm[8];
-  const int c = blockIdx.x, b = blockIdx.y;
-  const int n = req_len(seq_lens, max_seq_len, b);
-  const int k = req_k(k_per_seg, max_k, b, n);
-  if (c * kChunk >= n || k <= 0 || k == n) return;
-  low[threadIdx.x] = 0;
-  const uint32_t bin0 = w.state[b].bin0, want1 = w.state[b].want1;
-  uint32_t bin1, want2;
-  scan_hist12(w.hist1 + (int64_t)b * kBins12, want1, &bin1, &want2, sm);
-  if (c == 0 && threadIdx.x == 0) {
-    w.state[b].bin1 = bin1;
-    w.state[b].want2 = want2;
-  }
-  const uint32_t prefix = (bin0 << 12) | bin1;
-  uint32_t key[16], valid;
-  load_chunk_keys<false>(scores + (int64_t)b * score_stride, n, c, key, valid);
-  uint32_t gt = 0;
-#pragma unroll
-  for (int j = 0; j < 16; ++j) {
-    if (!(valid >> j & 1)) continue;
-    const uint32_t hi = key[j] >> 8;
-    if ((hi >> 12) == bin0 && hi > prefix) ++gt;
-    else if (hi == prefix) atomicAdd(&low[key[j] & 0xffu], 1u);
-  }
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) gt += __shfl_xor(gt, o);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = gt;
-  __syncthreads();
-  if (threadIdx.x == 0) w.chunk_gt[(int64_t)b * w.max_chunks + c] += sm[0] + sm[1] + sm[2] + sm[3];
-  w.chunk_low[((int64_t)b * w.max_chunks + c) * 256 + threadIdx.x] = (uint16_t)low[threadIdx.x];
-}
-
-__global__ __launch_bounds__(kMbThreads) void topk_mb_pass4(const float* __restrict__ scores,
+__global__ __launch_bounds__(kMbThreads) void topk_mb_write(const float* __restrict__ scores,
                                                             int64_t score_stride,
                                                             const int32_t* __restrict__ seq_lens,
                                                             int max_seq_len,
@@ -274,102 +360,172 @@ __global__ __launch_bounds__(kMbThreads) void topk_mb_pass4(const float* __restr
                                                             int max_k, TopkMbWs w,
                                                             int32_t* __restrict__ idx_out,
                                                             int64_t idx_stride) {
-  __shared__ uint32_t sm[16];
+  __shared__ __attribute__((aligned(16))) uint32_t hA[1024], hB[1024], hBb[1024];
+  __shared__ uint32_t cache[kCandCache];
+  __shared__ uint32_t sm[8];
+  __shared__ uint32_t acc;                 // selected keys of the chunks before this one, above T
+  __shared__ uint32_t part[2][kMbWaves];   // wave totals of the compaction, alternating per tile
   const int c = blockIdx.x, b = blockIdx.y, t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int n = req_len(seq_lens, max_seq_len, b);
   const int k = req_k(k_per_seg, max_k, b, n);
-  if (c * kChunk >= n || k <= 0) return;
+  const int tile0 = c * w.chunk_tiles;
+  if ((int64_t)tile0 * kTile >= n || k <= 0) return;
+  const int chunk_keys = w.chunk_tiles * kTile;
   int32_t* out = idx_out + (int64_t)b * idx_stride;
   if (k == n) {  // everything is selected
-    for (int i = c * kChunk + t; i < n && i < (c + 1) * kChunk; i += kMbThreads) out[i] = i;
+    const int hi = (c + 1) * chunk_keys < n ? (c + 1) * chunk_keys : n;
+    for (int i = c * chunk_keys + t; i < hi; i += kMbThreads) out[i] = i;
     return;
   }
-  const int chunks = (n + kChunk - 1) / kChunk;
   const TopkMbState st = w.state[b];
-  // column t of the per-chunk low-byte histograms: over all chunks, and over those before c
-  uint32_t total = 0, before = 0;
-  const uint16_t* col = w.chunk_low + (int64_t)b * w.max_chunks * 256 + t;
-#pragma unroll 4
-  for (int x = 0; x < chunks; ++x) {
-    const uint32_t v = col[(int64_t)x * 256];
-    total += v;
-    if (x < c) before += v;
-  }
-  // suffix scan over the 256 low-byte values (thread t holds value t): rank from the top
-  uint32_t inc = total;  // inclusive sum over values >= t within the wave, built from the high end
-#pragma unroll
-  for (int o = 1; o < 64; o <<= 1) {
-    const uint32_t v = __shfl_down(inc, o);
-    if (lane + o < 64) inc += v;
-  }
-  if (lane == 0) sm[wave] = inc;
+  // the chunk's first tile is requested now and used once the threshold is known
+  const float* s = scores + (int64_t)b * score_stride;
+  float x[4];
+  uint32_t valid;
+  load_tile_raw(s, n, tile0, x, valid);
+  const uint32_t M = st.num_cand < (uint32_t)n ? st.num_cand : (uint32_t)n;  // candidates of the request
+  const uint32_t Mb = w.cand_base[(int64_t)b * w.max_chunks + c];            // ... of the chunks before this one
+  uint32_t gt_before = 0;  // this thread's share of the keys above T in the chunks before this one
+  for (int i = t; i < c * kMbWaves; i += kMbThreads) gt_before += w.chunk_gt[(int64_t)b * w.max_chunks * kMbWaves + i];
+  hA[t] = hB[t] = hBb[t] = 0;
+  if (t == 0) acc = 0;
   __syncthreads();
-  uint32_t above_waves = 0;
-  for (int x = wave + 1; x < 4; ++x) above_waves += sm[x];
-  inc += above_waves;                  // keys of the prefix with low byte >= t
-  const uint32_t exc = inc - total;    // ... with low byte > t
-  __syncthreads();
-  if (exc < st.want2 && st.want2 <= inc) {  // exactly one thread: its value is T's low byte
-    sm[8] = (uint32_t)t;
-    sm[9] = st.want2 - exc;  // how many keys == T are taken
-  }
-  __syncthreads();
-  const uint32_t low_t = sm[8], need_eq = sm[9];
-  const uint32_t T = (st.bin0 << 20) | (st.bin1 << 8) | low_t;
-  // selected keys in the chunks before this one: above the prefix, inside it above T, equal to T
-  uint32_t gt_before = (t > (int)low_t) ? before : 0u;
-  for (int x = t; x < c; x += kMbThreads) gt_before += w.chunk_gt[(int64_t)b * w.max_chunks + x];
-  uint32_t eq_before = (t == (int)low_t) ? before : 0u;
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) {
-    gt_before += __shfl_xor(gt_before, o);
-    eq_before += __shfl_xor(eq_before, o);
-  }
-  __syncthreads();
-  if (lane == 0) {
-    sm[wave] = gt_before;
-    sm[4 + wave] = eq_before;
-  }
-  __syncthreads();
-  gt_before = sm[0] + sm[1] + sm[2] + sm[3];
-  eq_before = sm[4] + sm[5] + sm[6] + sm[7];
-  __syncthreads();
+  const bool cached = M <= (uint32_t)kCandCache;
+  const uint32_t* cand = w.cand + (int64_t)b * w.max_chunks * chunk_keys;
 
-  // ordered compaction of this chunk: 16 consecutive tokens per thread
-  uint32_t key[16], valid;
-  load_chunk_keys<true>(scores + (int64_t)b * score_stride, n, c, key, valid);
-  uint32_t gmask = 0, emask = 0;
+  // level A: bits 19..10 of all candidates, four loads per thread in flight
+  for (uint32_t base = 0; base < M; base += 4 * kMbThreads) {
+    uint32_t kk[4];
 #pragma unroll
-  for (int j = 0; j < 16; ++j) {
-    if (!(valid >> j & 1)) continue;
-    if (key[j] > T) gmask |= 1u << j;
-    else if (key[j] == T) emask |= 1u << j;
-  }
-  const uint32_t packed = __popc(gmask) | (__popc(emask) << 16);  // <= 4096 each per chunk
-  uint32_t pinc = packed;
-#pragma unroll
-  for (int o = 1; o < 64; o <<= 1) {
-    const uint32_t v = __shfl_up(pinc, o);
-    if (lane >= o) pinc += v;
-  }
-  if (lane == 63) sm[wave] = pinc;
-  __syncthreads();
-  uint32_t woff = 0;
-  for (int x = 0; x < wave; ++x) woff += sm[x];
-  const uint32_t pexc = pinc - packed + woff;
-  uint32_t pgt = gt_before + (pexc & 0xffffu);
-  uint32_t peq = eq_before + (pexc >> 16);
-  const int i0 = c * kChunk + 16 * t;
-#pragma unroll
-  for (int j = 0; j < 16; ++j) {
-    if (gmask >> j & 1) {
-      const uint32_t pos = pgt + (peq < need_eq ? peq : need_eq);
-      if (pos < (uint32_t)k) out[pos] = i0 + j;  // the bound only matters if the counts were corrupted
-      ++pgt;
-    } else if (emask >> j & 1) {
-      if (peq < need_eq && pgt + peq < (uint32_t)k) out[pgt + peq] = i0 + j;
-      ++peq;
+    for (int u = 0; u < 4; ++u) {
+      const uint32_t i = base + u * kMbThreads + t;
+      kk[u] = i < M ? cand[i] : 0u;
     }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uint32_t i = base + u * kMbThreads + t;
+      if (i < M) {
+        if (cached) cache[i] = kk[u];
+        atomicAdd(&hA[(kk[u] >> 10) & 1023u], 1u);
+      }
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    uint32_t ba, wb;
+    wave_find_bin<1024>(hA, st.want1, ba, wb);
+    if (lane == 0) {
+      sm[0] = ba;
+      sm[1] = wb;
+    }
+  }
+  __syncthreads();
+  const uint32_t binA = sm[0], wantB = sm[1];
+
+  // level B: bits 9..0 of the candidates inside bin A, over all chunks and over the chunks before
+  // this one; candidates of earlier chunks in higher A bins are above T whatever T's low bits
+  {
+    auto visit = [&](uint32_t i, uint32_t kk) {
+      const uint32_t a = (kk >> 10) & 1023u;
+      if (a == binA) {
+        atomicAdd(&hB[kk & 1023u], 1u);
+        if (i < Mb) atomicAdd(&hBb[kk & 1023u], 1u);
+      } else if (a > binA && i < Mb) {
+        ++gt_before;
+      }
+    };
+    if (cached) {
+      for (uint32_t i = t; i < M; i += kMbThreads) visit(i, cache[i]);
+    } else {
+      for (uint32_t base = 0; base < M; base += 4 * kMbThreads) {
+        uint32_t kk[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const uint32_t i = base + u * kMbThreads + t;
+          kk[u] = i < M ? cand[i] : 0u;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const uint32_t i = base + u * kMbThreads + t;
+          if (i < M) visit(i, kk[u]);
+        }
+      }
+    }
+  }
+  gt_before = wave_sum(gt_before);
+  if (lane == 0 && gt_before) atomicAdd(&acc, gt_before);
+  __syncthreads();
+  if (wave == 0) {
+    uint32_t bb, ne;
+    wave_find_bin<1024>(hB, wantB, bb, ne);
+    // keys of the earlier chunks inside bin A: above T's low bits, and equal to them
+    uint32_t g = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int first = 1024 - 16 * (lane + 1) + 4 * q;
+      const uint4 v = *reinterpret_cast<const uint4*>(hBb + first);
+      if ((uint32_t)first > bb) g += v.x;
+      if ((uint32_t)first + 1 > bb) g += v.y;
+      if ((uint32_t)first + 2 > bb) g += v.z;
+      if ((uint32_t)first + 3 > bb) g += v.w;
+    }
+    g = wave_sum(g);
+    if (lane == 0) {
+      sm[2] = bb;
+      sm[3] = ne;
+      sm[4] = hBb[bb];
+      sm[5] = acc + g;
+    }
+  }
+  __syncthreads();
+  const uint32_t binB = sm[2], need_eq = sm[3], eq_before = sm[4];
+  gt_before = sm[5];
+  const uint32_t T = (st.bin0 << 20) | (binA << 10) | binB;
+
+  // ordered compaction of this chunk, tile after tile: 4 consecutive tokens per thread
+  uint32_t run_gt = gt_before, run_eq = eq_before;
+  for (int i = 0;;) {
+    uint32_t key[4];
+    keys_of(x, key);
+    uint32_t gmask = 0, emask = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (!(valid >> j & 1)) continue;
+      if (key[j] > T) gmask |= 1u << j;
+      else if (key[j] == T) emask |= 1u << j;
+    }
+    const uint32_t packed = __popc(gmask) | (__popc(emask) << 16);  // <= 4096 each per tile
+    const uint32_t pinc = wave_scan(packed);
+    if (lane == 63) part[i & 1][wave] = pinc;
+    __syncthreads();
+    // wave totals -> offsets: lanes 0..15 of every wave scan the sixteen totals
+    uint32_t tinc = part[i & 1][lane & 15];
+    const uint32_t tmine = tinc;
+#pragma unroll
+    for (int o = 1; o < 16; o <<= 1) {
+      const uint32_t u = __shfl_up(tinc, o, 16);
+      if ((lane & 15) >= o) tinc += u;
+    }
+    const uint32_t woff = __shfl(tinc - tmine, wave), total = __shfl(tinc, 15);
+    const uint32_t pexc = pinc - packed + woff;
+    uint32_t pgt = run_gt + (pexc & 0xffffu);
+    uint32_t peq = run_eq + (pexc >> 16);
+    const int i0 = (tile0 + i) * kTile + 4 * t;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (gmask >> j & 1) {
+        const uint32_t pos = pgt + (peq < need_eq ? peq : need_eq);
+        if (pos < (uint32_t)k) out[pos] = i0 + j;  // the bound only matters if the counts were corrupted
+        ++pgt;
+      } else if (emask >> j & 1) {
+        if (peq < need_eq && pgt + peq < (uint32_t)k) out[pgt + peq] = i0 + j;
+        ++peq;
+      }
+    }
+    run_gt += total & 0xffffu;
+    run_eq += total >> 16;
+    if (++i >= w.chunk_tiles || (int64_t)(tile0 + i) * kTile >= n) break;
+    load_tile_raw(s, n, tile0 + i, x, valid);
   }
 }
 
@@ -378,16 +534,11 @@ int launch_topk_mb(const float* scores, int64_t score_stride, const int32_t* seq
                    int32_t* idx_out, int64_t idx_stride, void* ws, hipStream_t stream) {
   const TopkMbWs w = carve_topk(ws, batch, max_seq_len);
   dim3 grid(w.max_chunks, batch), block(kMbThreads);
-  const int n16 = batch * kBins12 * 2 * 4 / 16;  // hist0 and hist1 are adjacent
-  hipLaunchKernelGGL(topk_mb_pass0, dim3((n16 + kMbThreads - 1) / kMbThreads), block, 0, stream,
-                     reinterpret_cast<uint4*>(w.hist0), n16);
-  hipLaunchKernelGGL(topk_mb_pass1, grid, block, 0, stream, scores, score_stride, seq_lens,
+  hipLaunchKernelGGL(topk_mb_hist, grid, block, 0, stream, scores, score_stride, seq_lens,
                      max_seq_len, k_per_seg, max_k, w);
-  hipLaunchKernelGGL(topk_mb_pass2, grid, block, 0, stream, scores, score_stride, seq_lens,
+  hipLaunchKernelGGL(topk_mb_cand, grid, block, 0, stream, scores, score_stride, seq_lens,
                      max_seq_len, k_per_seg, max_k, w);
-  hipLaunchKernelGGL(topk_mb_pass3, grid, block, 0, stream, scores, score_stride, seq_lens,
-                     max_seq_len, k_per_seg, max_k, w);
-  hipLaunchKernelGGL(topk_mb_pass4, grid, block, 0, stream, scores, score_stride, seq_lens,
+  hipLaunchKernelGGL(topk_mb_write, grid, block, 0, stream, scores, score_stride, seq_lens,
                      max_seq_len, k_per_seg, max_k, w, idx_out, idx_stride);
   OKV_HIP_CHECK(hipGetLastError());
   return OKV_OK;

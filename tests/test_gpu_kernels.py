@@ -245,7 +245,7 @@ def _topk_single_workgroup(scores_dev, k):
     return out
 
 
-@pytest.mark.parametrize("n", [16384, 16385, 40000, 131072 + 3])
+@pytest.mark.parametrize("n", [14336, 14337, 16385, 40000, 131072 + 3])
 def test_topk_long_special_values_and_both_kernels(n):
     g = torch.Generator().manual_seed(n)
     s = torch.randn((2, n), generator=g)
@@ -273,6 +273,27 @@ def test_topk_repeated_calls_leave_workspace_clean():
         if i % 2:
             s = torch.softmax(s * 3, dim=-1)
         _check_topk(s, max(1, int(0.067 * n)))
+
+
+def test_topk_multi_tile_chunks_and_many_candidates():
+    """Lengths whose chunks hold several tiles (2 at 450K; the 15-tile cap and more than 64 chunks
+    at 4.2M), and score sets whose threshold bin holds more candidates than the last launch
+    caches in LDS (a few distinct values; a narrow band), checked against the stable sort."""
+    g = torch.Generator().manual_seed(5)
+    for n in (450000, 4_200_000):
+        s = torch.randn((1, n), generator=g)
+        _check_topk(s, int(0.067 * n))
+        _check_topk(torch.round(s * 2) / 2, int(0.067 * n))            # ~10 distinct values
+        _check_topk(1.0 + s * 1e-3, n // 3)                              # everything inside one level-0 bin
+    s = torch.randn((3, 300000), generator=g)
+    s[1] = torch.round(s[1] * 8) / 8
+    lens = torch.tensor([300000, 262145, 4097], dtype=torch.int32)
+    kper = torch.tensor([20000, 262144, 4097], dtype=torch.int32)
+    out = torch.full((3, 262144), -1, dtype=torch.int32, device=DEV)
+    ops.topk(s.to(DEV), 262144, seq_lens=lens.to(DEV), k_per_seg=kper.to(DEV), out=out)
+    for b in range(3):
+        want = orc.select_topk_stable(s[b:b + 1, :int(lens[b])], int(kper[b]))[0]
+        assert torch.equal(out[b, :int(kper[b])].cpu().to(torch.int64), want), b
 
 
 # ------------------------------------------------------------------ window selectors
