@@ -273,7 +273,7 @@ __device__ __forceinline__ void finish_body(const RowList& rows, int hq, const A
           for (int u = 0; u < U; ++u) {
             const float mn = fmaxf(M, xs[u]);
             if (mn != -INFINITY) {
-              d = fmaf(d, exp2f(M - mn), exp2f(xs[u] - mn));
+              d = fmaf(d, __builtin_amdgcn_exp2f(M - mn), __builtin_amdgcn_exp2f(xs[u] - mn));
               M = mn;
             }
           }
@@ -283,7 +283,7 @@ __device__ __forceinline__ void finish_body(const RowList& rows, int hq, const A
       for (int o = 1; o < 8; o <<= 1) {
         const float M2 = __shfl_xor(M, o), d2 = __shfl_xor(d, o);
         const float mn = fmaxf(M, M2);
-        if (mn != -INFINITY) d = d * exp2f(M - mn) + d2 * exp2f(M2 - mn);
+        if (mn != -INFINITY) d = d * __builtin_amdgcn_exp2f(M - mn) + d2 * __builtin_amdgcn_exp2f(M2 - mn);
         M = mn;
       }
       if (h < hq && sub == 0) s_lse[h] = M + log2f(d);
@@ -302,7 +302,9 @@ __device__ __forceinline__ void finish_body(const RowList& rows, int hq, const A
     const float lse = soft ? (own_lse ? s_lse[h] : w.score_lse[b * hq + h]) : 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      float x = soft ? exp2f(v[i] * kLog2e - lse) : v[i];
+      // one v_exp_f32 (a probability below 2^-126 counts as zero): with Hq exponentials per token
+      // the block's time was its arithmetic, not its loads
+      float x = soft ? __builtin_amdgcn_exp2f(fmaf(v[i], kLog2e, -lse)) : v[i];
       acc[i] = is_max ? fmaxf(acc[i], x) : acc[i] + x;
     }
   }
