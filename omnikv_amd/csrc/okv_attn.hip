@@ -82,8 +82,8 @@ __global__ __launch_bounds__(256) void attn_stage1_generic(const T* __restrict__
     for (int h = 0; h < G; ++h) {
       float s2 = s[h] * sl2;
       float mn = fmaxf(m[h], s2);
-      float alpha = exp2f(m[h] - mn);
-      float p = exp2f(s2 - mn);
+      float alpha = __builtin_amdgcn_exp2f(m[h] - mn);
+      float p = __builtin_amdgcn_exp2f(s2 - mn);
       l[h] = l[h] * alpha + p;
       m[h] = mn;
       if (WITH_V) {
@@ -188,7 +188,7 @@ __device__ __forceinline__ void merge_body(const RowList& rows, int hq, const At
       if (s >= ns) break;
       const float x = xs[u];
       const float mn = fmaxf(m, x);
-      const float a = exp2f(m - mn), f = exp2f(x - mn);
+      const float a = __builtin_amdgcn_exp2f(m - mn), f = __builtin_amdgcn_exp2f(x - mn);
       den = fmaf(den, a, f);
       num.x = fmaf(num.x, a, f * os[u].x);
       num.y = fmaf(num.y, a, f * os[u].y);
