@@ -34,28 +34,28 @@ static int num_compute_units() {
   return cus;
 }
 
-// Rows per split.  The pass is bandwidth-bound, so the grid is sized to what the
-// chip holds at once (resident workgroups per CU: 3 with V, 6 for scoring alone),
-// every workgroup getting the same share of rows: all of them start together and
-// finish together, in one round when the split fits the row cap, else in the fewest
-// equal rounds.  The cap keeps the LDS staging of a scored split's logits small.
+// Rows per split.  The pass is bandwidth-bound, so the grid is sized to what the chip holds at
+// once, every workgroup getting the same share of rows: all of them start together and finish
+// together, in one round when the split fits the row cap, else in the fewest equal rounds.
+// The attention kernels hold two workgroups per CU (their registers allow two waves per SIMD),
+// scoring alone six.  The cap keeps the LDS staging of a scored split's logits small.
 static int choose_split_rows(int batch, int hq, int hkv, int total_rows, bool with_v,
                              bool with_logits, bool gather) {
   if (g_split_rows_override > 0) return g_split_rows_override;
-  // workgroups the chip runs side by side: the gather pass (selected rows through an index) is
-  // a chain of latencies and does best in exactly one round of two per CU -- measured: 192
-  // rows at 8781 selected rows, 512 at 30150; the streaming passes in 1.5 rounds of three
-  // (a batch is sized by its longest request, so ragged ones fill less than that: three there too)
-  const int64_t capacity = (int64_t)num_compute_units() * (gather && batch <= 1 ? 2 : with_v ? 3 : 6);
-  // a scored split stages G*rows fp32 logits in LDS: keep that within 32 KB
+  (void)gather;
+  // a batch is sized by its longest request, so ragged ones fill less than the grid suggests:
+  // three per CU there (measured on 16 requests of 8K..32K tokens)
+  const int64_t capacity = (int64_t)num_compute_units() * (with_v ? (batch <= 1 ? 2 : 3) : 6);
+  // a scored split stages G*rows fp32 logits in LDS: keep that within 33 KB (2112 rows at G = 4,
+  // what one round of a 128K context needs)
   const int group = hkv > 0 && hq >= hkv ? hq / hkv : 1;
-  const int64_t cap_rows = with_logits ? (8192 / group) / 64 * 64 : 4096;
+  const int64_t cap_rows = with_logits ? (8448 / group) / 64 * 64 : 4096;
   const int64_t work = (int64_t)(total_rows > 0 ? total_rows : 1) * hkv * (batch > 0 ? batch : 1);
   for (int64_t rounds = 1;; ++rounds) {
     int64_t rows = (work + rounds * capacity - 1) / (rounds * capacity);
     rows = (rows + 63) / 64 * 64;
-    if (rounds == 1 && with_v && !(gather && batch <= 1) && rows <= 128) {
-      // a short dense pass is a latency chain too: fewer, fatter workgroups
+    if (rounds == 1 && with_v && batch > 1 && rows <= 128) {
+      // a short pass is a chain of latencies: fewer, fatter workgroups
       rows = (work + capacity * 2 / 3 - 1) / (capacity * 2 / 3);
       rows = (rows + 63) / 64 * 64;
     }
