@@ -37,15 +37,16 @@ static int num_compute_units() {
 // Rows per split.  The pass is bandwidth-bound, so the grid is sized to what the chip holds at
 // once, every workgroup getting the same share of rows: all of them start together and finish
 // together, in one round when the split fits the row cap, else in the fewest equal rounds.
-// The attention kernels hold two workgroups per CU (their registers allow two waves per SIMD),
-// scoring alone six.  The cap keeps the LDS staging of a scored split's logits small.
+// The attention kernels hold two workgroups per CU (their registers allow two waves per SIMD);
+// scoring alone could hold five and does best sized for three (measured at 128K: 50.6 us against
+// 53.1 sized for six).  The cap keeps the LDS staging of a scored split's logits small.
 static int choose_split_rows(int batch, int hq, int hkv, int total_rows, bool with_v,
                              bool with_logits, bool gather) {
   if (g_split_rows_override > 0) return g_split_rows_override;
   (void)gather;
   // a batch is sized by its longest request, so ragged ones fill less than the grid suggests:
-  // three per CU there (measured on 16 requests of 8K..32K tokens)
-  const int64_t capacity = (int64_t)num_compute_units() * (with_v ? (batch <= 1 ? 2 : 3) : 6);
+  // three and six per CU there (measured on 16 requests of 8K..32K tokens)
+  const int64_t capacity = (int64_t)num_compute_units() * (batch <= 1 ? (with_v ? 2 : 3) : (with_v ? 3 : 6));
   // a scored split stages G*rows fp32 logits in LDS: keep that within 33 KB (2112 rows at G = 4,
   // what one round of a 128K context needs)
   const int group = hkv > 0 && hq >= hkv ? hq / hkv : 1;
