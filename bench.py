@@ -236,6 +236,19 @@ def main():
         stream.synchronize()
         wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
+        # ---- spread of single steps (outside the timed region): one event pair per step
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+               for _ in range(max(args.steps, 20))]
+        for e0, e1 in evs:
+            e0.record(stream)
+            run()
+            e1.record(stream)
+        stream.synchronize()
+        per_step = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
+
+        def pct(p):
+            return per_step[min(len(per_step) - 1, int(p * len(per_step)))]
+
         # ---- dominant kernel: dense split attention over N+tail rows, eager, events
         dense_layers = [l for l, kd in schedule().items() if kd[0] == "dense"]
         reps = 10
@@ -305,6 +318,7 @@ def main():
         },
         "decode_tokens_per_s_attention_only": 1e3 / wall_ms,
         "step_hbm_gbs": step_bytes / (wall_ms * 1e-3) / 1e9,
+        "step_ms_p10_p50_p90": [round(pct(0.1), 4), round(pct(0.5), 4), round(pct(0.9), 4)],
         "roofline": {
             "kernel": "okv::attn_stage1_mfma<BF16,4,true,0,false> (dense split pass over N+tail rows of K and V)"
             if dtype != torch.float32 else "okv::attn_stage1_generic<float,4,true> (dense split pass)",
