@@ -211,7 +211,7 @@ __device__ __forceinline__ float quad_swap(float x) {
 // grid (row blocks, batch), one wave per kv head; LDS: [window][rows_per_block + 1] bit
 // patterns of non-negative floats (their unsigned order is their numeric order).
 template <typename T, int NCB>
-__global__ __launch_bounds__(512) void window_score_mfma(WindowArgs a, int rows_per_block, int exp_decay,
+__global__ __launch_bounds__(512, 4) void window_score_mfma(WindowArgs a, int rows_per_block, int exp_decay,
                                                          float* __restrict__ scores,
                                                          int64_t score_stride) {
   extern __shared__ uint32_t wmax[];
@@ -272,18 +272,19 @@ __global__ __launch_bounds__(512) void window_score_mfma(WindowArgs a, int rows_
   };
   __syncthreads();  // the zero fill is complete
   {
-    // four tiles in flight per wave (one workgroup per CU has to cover the memory latency
-    // by itself); every load is unconditional, past the end it repeats the last tile
-    uint4 kf[4][4];
+    // two tiles in flight per wave and 128 registers at most, so that two workgroups fit a CU
+    // (four waves per SIMD: 58 us at 128K against 66 us for one workgroup with four tiles in
+    // flight); every load is unconditional, past the end it repeats the last tile
+    uint4 kf[2][4];
     const int t_last = begin + ((last - begin) >> 4 << 4);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) load_tile(min(begin + 16 * u, t_last), kf[u]);
-    for (int t = begin; t <= t_last; t += 64) {
+    for (int u = 0; u < 2; ++u) load_tile(min(begin + 16 * u, t_last), kf[u]);
+    for (int t = begin; t <= t_last; t += 32) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < 2; ++u) {
         const int tt = t + 16 * u;
         if (tt <= t_last) compute(tt, kf[u]);
-        load_tile(min(tt + 64, t_last), kf[u]);
+        load_tile(min(tt + 32, t_last), kf[u]);
       }
     }
   }
@@ -328,8 +329,8 @@ static void launch_window(WindowArgs a, int batch, int exp_decay, float* scores,
                           int cus, hipStream_t stream) {
   hipLaunchKernelGGL((window_lse_mfma<T, NCB>), dim3(a.hkv, a.max_splits, batch), dim3(256), 0, stream, a);
   hipLaunchKernelGGL(window_lse_merge, dim3(batch * a.hkv), dim3(256), 0, stream, a);
-  // one round of row blocks, one block of `hkv` waves per CU; LDS bounds the rows
-  int64_t per = ((int64_t)a.max_score_len * batch + cus - 1) / cus;
+  // one round of row blocks, two blocks of `hkv` waves per CU; LDS bounds the rows
+  int64_t per = ((int64_t)a.max_score_len * batch + 2 * cus - 1) / (2 * cus);
   int rpb = (int)((per + 15) / 16 * 16);
   if (rpb < 64) rpb = 64;
   const int cap = (48 * 1024 / 4 / a.window) / 16 * 16;
