@@ -84,6 +84,20 @@ def test_library_exports_every_declared_symbol():
     assert lib.okv_strerror(-3) == b"workspace too small"
 
 
+def test_header_is_plain_c(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 and as C++ with nothing but the
+    standard headers (no torch, no HIP types in the signatures)."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "hdr.c"
+    src.write_text('#include "omnikv_hip.h"\nint main(void) { okv_shape_t s; (void)s; return OKV_OK; }\n')
+    inc = os.path.join(ROOT, "include")
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-I", inc, str(src)])
+    subprocess.check_call(["g++", "-std=c++11", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", "-I", inc, str(src)])
+
+
 def test_workspace_sizes_are_consistent():
     base = ops.workspace_bytes(_lib.OKV_OP_DENSE_ATTN, 1, 32, 8, 128, 131072)
     with_scores = ops.workspace_bytes(_lib.OKV_OP_DENSE_ATTN, 1, 32, 8, 128, 131072, with_scores=True)
