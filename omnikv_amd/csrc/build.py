@@ -42,6 +42,23 @@ def build(force: bool = True, verbose: bool = True) -> str:
     return OUT
 
 
+ABI_SMOKE_SRC = os.path.join(os.path.dirname(PKG), "tests", "native", "abi_smoke.cpp")
+ABI_SMOKE_BIN = os.path.join(os.path.dirname(PKG), "tests", "native", "abi_smoke")
+
+
+def build_abi_smoke(verbose: bool = True) -> str:
+    """The host-only C++ program that exercises the C ABI without Python (tests/native/)."""
+    cmd = ["hipcc", "-O1", "-std=c++17", "-Wno-unused-command-line-argument", ABI_SMOKE_SRC, "-L", PKG,
+           "-lomnikv_hip", "-Wl,-rpath,$ORIGIN/../../omnikv_amd", "-o", ABI_SMOKE_BIN]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + res.stdout)
+    return ABI_SMOKE_BIN
+
+
 if __name__ == "__main__":
     build(force=True)
     print("built", OUT)
+    print("built", build_abi_smoke())

@@ -525,3 +525,16 @@ def test_topk_random_lengths_and_distributions_bit_exact():
             want = orc.select_topk_stable(s[b:b + 1, :lb], kb)[0]
             assert torch.equal(out[b, :kb].cpu().to(torch.int64), want), (case, b, lb, kb)
             assert (out[b, kb:] == -1).all()
+
+
+def test_c_abi_from_a_native_host_program():
+    """tests/native/abi_smoke.cpp (built beforehand next to its source) links the library, owns
+    its device memory through the HIP runtime, and checks scores, selection, dense and sparse
+    attention and the row gather against loops of its own: the C ABI needs no Python around it."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "native", "abi_smoke")
+    assert os.path.exists(exe), "build first: python -c 'import __graft_entry__ as g; g.build()'"
+    res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert res.returncode == 0, res.stdout
+    assert "abi smoke ok" in res.stdout
