@@ -538,3 +538,28 @@ def test_c_abi_from_a_native_host_program():
     res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
     assert res.returncode == 0, res.stdout
     assert "abi smoke ok" in res.stdout
+
+
+def test_topk_degenerate_score_vectors():
+    """Vectors made of one value, of two, of NaN, of infinities, of zeros of both signs, of
+    subnormals, and monotone ones: every key falls into one or two histogram bins, so the
+    selection is decided by the tie rule and the chunk offsets alone."""
+    n = 50021
+    cases = {
+        "all_nan": torch.full((1, n), float("nan")),
+        "all_inf": torch.full((1, n), float("inf")),
+        "all_ninf": torch.full((1, n), float("-inf")),
+        "all_negative": torch.full((1, n), -3.5),
+        "zeros_of_both_signs": torch.zeros((1, n)),
+        "every_other_nan": torch.randn((1, n), generator=torch.Generator().manual_seed(3)),
+        "subnormal": torch.randn((1, n), generator=torch.Generator().manual_seed(4)) * 1e-42,
+        "two_values": (torch.arange(n) % 2).float()[None],
+        "descending": torch.arange(n, 0, -1).float()[None],
+        "ascending": torch.arange(n).float()[None],
+    }
+    cases["zeros_of_both_signs"][0, ::2] = -0.0
+    cases["every_other_nan"][0, ::2] = float("nan")
+    for name, s in cases.items():
+        for k in (1, 7, 3351, n // 2, n - 1, n):
+            got = ops.topk(s.to(DEV), k).cpu().to(torch.int64)
+            assert torch.equal(got, orc.select_topk_stable(s, k)), (name, k)
