@@ -122,8 +122,9 @@ class OmniKVMultiStageCache:
         self._tail: Dict[int, _Store] = {}
         self._idx: Dict[int, torch.Tensor] = {}    # filter layer -> (bsz, k) int32 on the GPU
         self._part: Dict[int, torch.Tensor] = {}   # sparse layer -> (bsz, k, 2, Hkv, D) staged rows
-        self._part_src: Dict[int, int] = {}        # sparse layer -> id of the idx it was gathered with
-        self._staged_for: Dict[int, int] = {}      # sparse layer -> id of the idx its rows were staged with
+        self._sel_gen: Dict[int, int] = {}         # filter layer -> how many selections it has made
+        self._part_src: Dict[int, int] = {}        # sparse layer -> selection number it was gathered with
+        self._staged_for: Dict[int, int] = {}      # sparse layer -> selection number its rows were staged with
         self._staging: Dict[int, torch.Tensor] = {}
         self._events: Dict[int, torch.cuda.Event] = {}
         self._recorded: Dict[int, threading.Event] = {}
@@ -197,14 +198,41 @@ class OmniKVMultiStageCache:
         self._len32 = torch.tensor([n + 1], dtype=torch.int32, device=dev)
         self._tail_pos = torch.tensor([t0], dtype=torch.int64, device=dev)
         self._tail_len32 = torch.tensor([t0 + 1], dtype=torch.int32, device=dev)
+        # how many static steps the preallocated buffers take: every step writes one row at
+        # _pos into the dense stores and one at _tail_pos into the tails
+        dense_caps = [self._store[i].capacity for i, s in self.layer_state.items() if not s[0]]
+        tail_caps = [t.capacity for t in self._tail.values()]
+        self._static_caps = (min(dense_caps) if dense_caps else n + self.max_new_tokens,
+                             min(tail_caps) if tail_caps else t0 + self.max_new_tokens)
+        self._static_budget = min(self._static_caps[0] - n, self._static_caps[1] - t0)
+        self._static_steps = 0
         self._static = True
 
+    @property
+    def static_steps_left(self) -> int:
+        """Static decode steps (eager or graph replays) the preallocated buffers still take."""
+        return self._static_budget - self._static_steps
+
+    def note_static_step(self) -> None:
+        """Host-side count of static steps, taken BEFORE a step runs (each replay of a captured
+        step counts: the graph itself cannot).  The appends of a static step write at device
+        positions that nothing on the device checks, so running past the buffers must be
+        refused here."""
+        if self._static_steps >= self._static_budget:
+            raise RuntimeError(
+                f"static decode buffers are full after {self._static_steps} steps "
+                f"(max_new_tokens={self.max_new_tokens}): build the cache with a larger max_new_tokens")
+        self._static_steps += 1
+
     def advance_static(self) -> None:
-        """End of a static decode step: one more token everywhere (device-side adds)."""
-        self._pos += 1
-        self._len32 += 1
-        self._tail_pos += 1
-        self._tail_len32 += 1
+        """End of a static decode step: one more token everywhere (device-side adds).  The
+        positions stop at the last row of the buffers even if a caller replays a captured
+        step more often than note_static_step allows."""
+        dense_cap, tail_cap = self._static_caps
+        self._pos.add_(1).clamp_(max=dense_cap - 1)
+        self._len32.add_(1).clamp_(max=dense_cap)
+        self._tail_pos.add_(1).clamp_(max=tail_cap - 1)
+        self._tail_len32.add_(1).clamp_(max=tail_cap)
 
     def append(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int) -> None:
         """Store the new rows of `layer_idx` (what update() does before it returns;
@@ -239,6 +267,11 @@ class OmniKVMultiStageCache:
                 self._host_kv[layer_idx] = host
             elif host.shape[0] != n:
                 raise NotImplementedError("an offloaded layer takes its prompt in one prefill call")
+            if not key_states.is_cuda:  # rows that already live on the host (an adopted cache)
+                host[:, 0].copy_(key_states[0].permute(1, 0, 2))
+                host[:, 1].copy_(value_states[0].permute(1, 0, 2))
+                self._sync_lists(layer_idx)
+                return
             # device-to-host on a stream of its own: the next layer's prefill compute runs
             # meanwhile; the stream is drained when decoding starts (_finish_prefill_offload)
             cur = torch.cuda.current_stream(key_states.device)
@@ -291,6 +324,7 @@ class OmniKVMultiStageCache:
                 self.num_skipped_selections += 1
                 return
         self._idx[sel_layer_idx] = idx32
+        self._sel_gen[sel_layer_idx] = self._sel_gen.get(sel_layer_idx, 0) + 1
         hi = self.layer_state[sel_layer_idx][2]
         lo = sel_layer_idx + self.num_wait_layers + 1
         for i in range(lo, hi):
@@ -306,7 +340,12 @@ class OmniKVMultiStageCache:
     def from_dynamic_cache(cache, full_attn_layers: List, num_hidden_layers, num_wait_load_layers=2,
                            real_offload=True, **kwargs):
         """modeling/spec_cache.py:371-385; `cache` is anything with key_cache /
-        value_cache lists (or transformers >= 4.54 `.layers[i].keys/.values`)."""
+        value_cache lists (or transformers >= 4.54 `.layers[i].keys/.values`), usually empty
+        (the reference adopts the fresh DynamicCache of the first forward, omnikv.py:339-341).
+        A populated cache is taken in as a prompt: its rows are COPIED into this cache's own
+        storage and tiered as the constructor arguments say -- with real_offload the
+        selected-rows-only layers go to pinned host memory whichever device they came on,
+        where the reference keeps the adopted tensors as they are."""
         c = kwargs.pop("_cls", OmniKVMultiStageCache)(full_attn_layers, num_hidden_layers, num_wait_load_layers,
                                                        real_offload, **kwargs)
         keys = getattr(cache, "key_cache", None)
@@ -315,7 +354,12 @@ class OmniKVMultiStageCache:
             keys = [l.keys for l in cache.layers if getattr(l, "keys", None) is not None]
             vals = [l.values for l in cache.layers if getattr(l, "values", None) is not None]
         seen = getattr(cache, "_seen_tokens", None)
+        on_gpu = [k.device for k in (keys or []) if k.is_cuda]
+        dev = on_gpu[0] if on_gpu else torch.device("cuda", torch.cuda.current_device())
         for i, (k, v) in enumerate(zip(keys or [], vals or [])):
+            to_host = c.real_offload and c.layer_state[i][0]
+            if not to_host:  # stays (or becomes) GPU resident
+                k, v = k.to(dev), v.to(dev)
             c.append(k, v, i)
         c._seen_tokens = seen if seen is not None else (keys[0].shape[-2] if keys else 0)
         return c
@@ -413,9 +457,9 @@ class OmniKVMultiStageCache:
     def _wait_part(self, layer_idx: int) -> torch.Tensor:
         """Staged rows of an offloaded layer, ordered behind their copy on the current stream."""
         sel = self.layer_state[layer_idx][1]
-        if not self._stage_at_selection and self._staged_for.get(layer_idx) != id(self._idx[sel]):
+        if not self._stage_at_selection and self._staged_for.get(layer_idx) != self._sel_gen[sel]:
             self._start_offload(self._idx[sel], [layer_idx])  # this layer only, now
-            self._staged_for[layer_idx] = id(self._idx[sel])
+            self._staged_for[layer_idx] = self._sel_gen[sel]
         self._recorded[layer_idx].wait()
         torch.cuda.current_stream(self._part[layer_idx].device).wait_event(self._events[layer_idx])
         return self._part[layer_idx]
@@ -425,7 +469,7 @@ class OmniKVMultiStageCache:
         """(bsz, Hkv, k, D) K and V rows of the current selection; gathers on first use."""
         sel = self.layer_state[layer_idx][1]
         idx32 = self._idx[sel]
-        if self._part_src.get(layer_idx) != id(idx32):
+        if self._part_src.get(layer_idx) != self._sel_gen[sel]:
             if self.real_offload:
                 part = self._wait_part(layer_idx)
                 pk = part[:, :, 0].permute(0, 2, 1, 3)
@@ -435,7 +479,7 @@ class OmniKVMultiStageCache:
                 pk = ops.gather_rows(kview, idx32)
                 pv = ops.gather_rows(vview, idx32)
             self.part_key[layer_idx], self.part_value[layer_idx] = pk, pv
-            self._part_src[layer_idx] = id(idx32)
+            self._part_src[layer_idx] = self._sel_gen[sel]
         return self.part_key[layer_idx], self.part_value[layer_idx]
 
     def _prefill_rows(self, layer_idx: int) -> int:
@@ -490,6 +534,7 @@ class OmniKVMultiStageCache:
                 buf = torch.empty((scores.shape[0], k), dtype=torch.int32, device=scores.device)
                 self._idx[layer_idx] = buf  # the sparse layers keep reading this very buffer
             ops.topk(scores, k, out=buf)
+            self._sel_gen[layer_idx] = self._sel_gen.get(layer_idx, 0) + 1  # same buffer, new selection
             if self.real_offload:
                 self._stage_static(layer_idx, buf)
             return out, buf

@@ -129,6 +129,7 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
   const T* pvb = reinterpret_cast<const T*>(rows.v_base) + (int64_t)g * rows.head_stride;
   const uint32_t ts = (uint32_t)rows.token_stride, tts = (uint32_t)rows.tail_token_stride;
   const int last = end - 1;
+  const bool tiles_aligned = (begin & 15) == 0;  // block-uniform; every tile base is begin + 16*i
 
   // ---- which rows a tile touches (issues the index / page-table loads)
   const int32_t* idx_row = rows.idx + (int64_t)b * rows.idx_stride;
@@ -141,9 +142,15 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
       if (MODE == 0) {
         tr.tok[x] = r;
       } else if (MODE == 3) {
-        // pages of 16k rows: the whole tile lies in one page, looked up once through the scalar unit
-        const int tb = __builtin_amdgcn_readfirstlane(tbase);
-        tr.tok[x] = rows.page_table[(int64_t)b * rows.page_table_stride + (tb >> rows.page_shift)];
+        // pages of 16k rows: a tile that starts on a multiple of 16 lies in one page, looked up
+        // once through the scalar unit.  The splits behind a scoring boundary that is not a
+        // multiple of 16 start wherever it is: their tiles straddle pages, one lookup per row.
+        if (tiles_aligned) {
+          const int tb = __builtin_amdgcn_readfirstlane(tbase);
+          tr.tok[x] = rows.page_table[(int64_t)b * rows.page_table_stride + (tb >> rows.page_shift)];
+        } else {
+          tr.tok[x] = rows.page_table[(int64_t)b * rows.page_table_stride + (r >> rows.page_shift)];
+        }
       } else if (MODE == 1) {  // branch-free: the index holds at least one entry per request
         int ri = r < main_len ? r : main_len - 1;
         ri = ri < 0 ? 0 : ri;  // a request with tail rows only

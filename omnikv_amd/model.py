@@ -193,6 +193,20 @@ class OmniKVMulModel(nn.Module):
         return self.norm(h)
 
 
+class StaticDecodeGraph:
+    """A captured decode step plus the host-side count of its replays: every replay appends one
+    row at a device position, so the replay that would run past the preallocated buffers raises
+    instead (the captured kernels themselves check nothing)."""
+
+    def __init__(self, graph: torch.cuda.CUDAGraph, cache: OmniKVMultiStageCache):
+        self.graph = graph
+        self.cache = cache
+
+    def replay(self) -> None:
+        self.cache.note_static_step()
+        self.graph.replay()
+
+
 class OmniKVMulLM(nn.Module):
     """modeling/omnikv.py:271-394: builds the cache on first use, keeps `stage`,
     runs the model, applies lm_head to the LAST position only, returns fp32 logits."""
@@ -230,6 +244,8 @@ class OmniKVMulLM(nn.Module):
         past_key_values.stage = "decoding" if n == 1 else "prefill"
         static = n == 1 and getattr(past_key_values, "_static", False)
         if static:
+            if not torch.cuda.is_current_stream_capturing():  # replays are counted by StaticDecodeGraph
+                past_key_values.note_static_step()
             position_ids = past_key_values._pos.view(1, 1).expand(input_ids.shape[0], -1)
         elif position_ids is None:
             start = past_key_values.get_seq_length()
@@ -266,7 +282,7 @@ class OmniKVMulLM(nn.Module):
                 logits, _ = self.forward(token, cache)
                 token.copy_(logits[:, -1].argmax(-1, keepdim=True))
         torch.cuda.current_stream(token.device).wait_stream(stream)
-        return graph, token, logits
+        return StaticDecodeGraph(graph, cache), token, logits
 
     @torch.no_grad()
     def generate_greedy(self, input_ids, num_tokens: int, **cache_kwargs) -> Tuple[torch.Tensor, List[torch.Tensor]]:

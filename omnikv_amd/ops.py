@@ -51,7 +51,8 @@ class PagedKV:
         if self.pool_k.stride(0) != self.page_size * self.pool_k.stride(1):
             raise ValueError("the pool's pages must lie back to back")
         t = idx.clamp(min=0).to(torch.int64)
-        slots = self.page_table.gather(1, t // self.page_size).to(torch.int64) * self.page_size + t % self.page_size
+        page = (t // self.page_size).clamp(max=self.page_table.shape[1] - 1)  # a stray entry never reads outside the table
+        slots = self.page_table.gather(1, page).to(torch.int64) * self.page_size + t % self.page_size
         return torch.where(idx < 0, idx, slots.to(torch.int32))
 
 
@@ -211,7 +212,10 @@ def topk(scores: torch.Tensor, k: int, seq_lens: Optional[torch.Tensor] = None,
     batch, n = scores.shape
     kk = min(k, n)
     if out is None:
-        out = torch.empty((batch, kk), dtype=torch.int32, device=scores.device)
+        if seq_lens is None and k_per_seg is None:
+            out = torch.empty((batch, kk), dtype=torch.int32, device=scores.device)
+        else:  # ragged: the kernels leave entries beyond a request's own k untouched -> padding is -1
+            out = torch.full((batch, kk), -1, dtype=torch.int32, device=scores.device)
     if kk == 0:
         return out
     ws = _workspace(scores.device, workspace_bytes(_lib.OKV_OP_TOPK, batch, 0, 0, 0, n))

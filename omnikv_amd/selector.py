@@ -27,10 +27,10 @@ def apply_rotary_pos_emb(q, k, cos, sin, unsqueeze_dim: int = 1):
     return q * cos + rotate_half(q) * sin, k * cos + rotate_half(k) * sin
 
 
-def select_from_query(query_states: torch.Tensor, key_cache: torch.Tensor, num_selected_tokens: int,
-                      consider_len: int, selector_cls: str = "last") -> torch.Tensor:
-    """query_states (bsz, Hq, Lq, D) already rotated; key_cache (bsz, Hkv, N, D) or an
-    ops.PagedKV.  Returns ascending int64 indices (bsz, min(k, consider_len))."""
+def score_from_query(query_states: torch.Tensor, key_cache: torch.Tensor, consider_len: int,
+                     selector_cls: str = "last") -> torch.Tensor:
+    """(bsz, consider_len) fp32 scores of the first consider_len cached tokens: the part of
+    modeling/omnikv.py:37-105 between the rotated query and the top-k."""
     if selector_cls in ops.SELECTOR_MODES:
         scores = ops.score(query_states[:, :, -1:, :], key_cache, score_len=consider_len, selector=selector_cls)
     elif selector_cls in ("uniform", "exp"):
@@ -50,6 +50,14 @@ def select_from_query(query_states: torch.Tensor, key_cache: torch.Tensor, num_s
                 scores = scores * 0.5 + s
     else:
         raise NotImplementedError(selector_cls)
+    return scores
+
+
+def select_from_query(query_states: torch.Tensor, key_cache: torch.Tensor, num_selected_tokens: int,
+                      consider_len: int, selector_cls: str = "last") -> torch.Tensor:
+    """query_states (bsz, Hq, Lq, D) already rotated; key_cache (bsz, Hkv, N, D) or an
+    ops.PagedKV.  Returns ascending int64 indices (bsz, min(k, consider_len))."""
+    scores = score_from_query(query_states, key_cache, consider_len, selector_cls)
     k = min(num_selected_tokens, scores.shape[-1])
     return ops.topk(scores, k).to(torch.int64)
 

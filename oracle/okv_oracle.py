@@ -25,6 +25,10 @@ How each function is pinned (tests/test_oracle_*.py):
     closed-form integer tables written out by hand from the reference loops.
   * gqa_attention               - torch scaled_dot_product_attention (library
     routine), fp64 explicit loops at tiny sizes, idx=all reduces to dense.
+  * score_tokens_by_kv_head, gqa_attention_by_kv_head - equal to the whole-tensor
+    functions to fp32 rounding (the matrix products see other shapes).
+  * paged_rows                  - scatter / gather round trip written with loops.
+  * lightllm_raw_head_max_score - sqrt(D) times the `last` score.
   * lse_merge                   - joint softmax over the concatenation.
   * OracleMultiStageCache       - element-wise comparison with index_select +
     cat written independently in the test.
@@ -114,6 +118,28 @@ def score_tokens(
                 s = torch.sum(s * alpha, dim=-2)
                 attn_sum = s if attn_sum is None else attn_sum * (2.0**-ql) + s
         return attn_sum
+    raise NotImplementedError(selector_cls)
+
+
+def score_tokens_by_kv_head(
+    q: torch.Tensor, k: torch.Tensor, consider_len: int, selector_cls: str = "last"
+) -> torch.Tensor:
+    """`score_tokens` of the `last` family evaluated one kv head at a time (the head
+    reduction is then max of maxes / sum of sums): the same arithmetic without the
+    4x repeated K of modeling/omnikv.py:38 held in memory at once, for the long
+    contexts.  Softmax is per q head, so splitting by head changes no per-head value;
+    only the order of the final additions over heads differs for the sum variant."""
+    hq, hkv = q.shape[1], k.shape[1]
+    g = hq // hkv
+    parts = [
+        score_tokens(q[:, g * i: g * (i + 1)], k[:, i: i + 1], consider_len, selector_cls)
+        for i in range(hkv)
+    ]
+    stack = torch.stack(parts, dim=0)
+    if selector_cls == "softmax_sum_last":
+        return stack.sum(dim=0)
+    if selector_cls in ("last", "softmax_before_last"):
+        return stack.max(dim=0).values
     raise NotImplementedError(selector_cls)
 
 
@@ -230,6 +256,16 @@ def gqa_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Te
     w = attn_logits(q, k)
     w = torch.nn.functional.softmax(w, dim=-1, dtype=torch.float32).to(q.dtype)
     return torch.matmul(w, repeat_kv(v, n_rep))
+
+
+def gqa_attention_by_kv_head(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+    """`gqa_attention` one kv head at a time (heads are independent: same values), so
+    that the repeated K and V of a 450K-token context are never held whole."""
+    g = q.shape[1] // k.shape[1]
+    return torch.cat(
+        [gqa_attention(q[:, g * i: g * (i + 1)], k[:, i: i + 1], v[:, i: i + 1]) for i in range(k.shape[1])],
+        dim=1,
+    )
 
 
 def attention_partial(

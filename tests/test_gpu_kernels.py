@@ -10,6 +10,7 @@ import torch
 
 from omnikv_amd import ops, synth
 from oracle import okv_oracle as orc
+from parity_helpers import assert_near_tie_only
 
 pytestmark = pytest.mark.gpu
 
@@ -116,11 +117,9 @@ def test_score_matches_oracle(selector, dtype, layout):
     assert _rel_err(got, want) < 1e-4
     if "softmax" in selector and "sum" in selector:
         assert abs(float(got.sum()) - 32.0) < 1e-2  # each head's softmax sums to one
-    # selected sets agree except for scores that differ in the last bits at the cut
+    # selected sets agree except for provable near-ties at the cut
     kk = orc.num_selected_tokens(0.067, n)
-    a = set(ops.topk(got.to(DEV), kk).cpu()[0].tolist())
-    b = set(orc.select_topk(want, kk)[0].tolist())
-    assert len(a & b) >= kk - 2
+    assert_near_tie_only(got[0], want[0], ops.topk(got.to(DEV), kk).cpu()[0], orc.select_topk_stable(want, kk)[0], kk)
 
 
 def test_score_partial_length_and_odd_sizes():
@@ -225,11 +224,14 @@ def test_filter_layer_op_config0(selector):
     out = ops.sparse_attn(qn.to(DEV), k2.to(DEV), v2.to(DEV), idx=idx)
     # identical fp32 scores -> identical indices
     assert torch.equal(ops.topk(scores_w.to(DEV), kk).cpu().to(torch.int64), idx_w)
-    # own scores: identical unless two scores at the cut differ only in the last bits
-    same = set(idx.cpu()[0].tolist()) & set(idx_w[0].tolist())
-    assert len(same) >= kk - 1
-    if len(same) == kk:
-        assert (out.cpu() - out_w[:, :, 0, :]).abs().max() < 1e-4
+    # own scores: identical up to provable near-ties at the cut
+    assert_near_tie_only(scores[0].cpu(), scores_w[0], idx.cpu()[0], idx_w[0], kk)
+    # the downstream layer on the ORACLE's rows, always; and on the kernel's own selection
+    # (one swapped near-tie row of 274 moves the output by far less than the tolerance)
+    out_on_oracle_idx = ops.sparse_attn(qn.to(DEV), k2.to(DEV), v2.to(DEV), idx=idx_w.to(torch.int32).to(DEV))
+    assert (out_on_oracle_idx.cpu() - out_w[:, :, 0, :]).abs().max() < 1e-4
+    own = orc.gqa_attention(qn, orc.gather_rows(k2, idx.cpu()[0].long()), orc.gather_rows(v2, idx.cpu()[0].long()))
+    assert (out.cpu() - own[:, :, 0, :]).abs().max() < 1e-4
 
 
 # ------------------------------------------------ long vectors: the chunked multi-workgroup path
@@ -320,9 +322,7 @@ def test_window_scores_match_oracle(selector, dtype, w, hq, hkv, n):
     assert got.shape == want.shape
     assert _rel_err(got, want) < 1e-4
     kk = max(1, int(0.067 * consider))
-    a = set(ops.topk(got.to(DEV), kk).cpu()[0].tolist())
-    b = set(orc.select_topk(want, kk)[0].tolist())
-    assert len(a & b) >= kk - 2
+    assert_near_tie_only(got[0], want[0], ops.topk(got.to(DEV), kk).cpu()[0], orc.select_topk_stable(want, kk)[0], kk)
 
 
 @pytest.mark.parametrize("selector", ["uniform", "exp"])

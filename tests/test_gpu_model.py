@@ -178,6 +178,28 @@ def test_graph_replayed_decode_matches_eager(selector_cls, offload):
             lm3.capture_decode(c3, tok)
 
 
+def test_static_decode_refuses_to_run_past_its_buffers():
+    """max_new_tokens rows are preallocated; the step that would write row max_new_tokens + 1
+    raises on the host (eager static steps and graph replays alike) and launches nothing."""
+    ids = torch.randint(0, SHAPE.vocab_size, (1, 200), generator=torch.Generator().manual_seed(6)).to(DEV)
+    lm = OmniKVMulLM(SHAPE, _config("last", False)).float().to(DEV)
+    lm.init_weights(seed=3, std=0.08)
+    budget = 6
+    logits, cache = lm.forward(ids, None, max_new_tokens=budget)
+    tok = logits[:, -1].argmax(-1, keepdim=True)
+    graph, token, _ = lm.capture_decode(cache, tok, warmup=2)
+    assert cache.static_steps_left == budget - 2
+    for _ in range(budget - 2):
+        graph.replay()
+    torch.cuda.synchronize()
+    assert cache.static_steps_left == 0
+    assert int(cache._pos) == 200 + budget - 1 and int(cache._len32) == 200 + budget  # clamped at the last row
+    with pytest.raises(RuntimeError, match="max_new_tokens"):
+        graph.replay()
+    with pytest.raises(RuntimeError, match="max_new_tokens"):
+        lm.forward(token, cache)
+
+
 def test_selection_tracing_compares_layers_and_leaves_decode_untouched(tmp_path):
     """Every layer reports what it would select (the reference's SAVE_SELECTED_IDX runs):
     the matrices are checked against the oracle's scores and stable top-k of the same

@@ -83,6 +83,52 @@ def test_paged_ragged_batch(page_size, dtype):
         assert float((raw[b, :n].cpu() - want).abs().max() / want.abs().max()) < 1e-4
 
 
+@pytest.mark.parametrize("page_size", [16, 64])
+def test_paged_scores_over_an_unaligned_prefix(page_size):
+    """The filter layer's decode step on a paged pool: scores over the prompt only, attention
+    over prompt + generated tokens.  The rows behind a scoring boundary that is not a multiple
+    of 16 are read in 16-row tiles that straddle pages."""
+    dtype = torch.bfloat16
+    lens = torch.tensor([2100, 133, 700, 4099, 64, 37], dtype=torch.int32)
+    cut = torch.tensor([37, 33, 1, 100, 16, 36], dtype=torch.int32)  # generated tokens per request
+    score_lens = lens - cut
+    q, ks, vs, pool_k, pool_v, table = _paged_batch(lens, page_size, dtype, seed=21)
+    kv = ops.PagedKV(pool_k.to(DEV), pool_v.to(DEV), table.to(DEV), page_size)
+    nmax, smax = int(lens.max()), int(score_lens.max())
+    for sel in ("last", "softmax_sum_last"):
+        out, scores = ops.dense_attn(q.to(DEV), kv, seq_len=nmax, seq_lens=lens.to(DEV), selector=sel,
+                                     score_len=smax, score_lens=score_lens.to(DEV))
+        for b, n in enumerate(int(x) for x in lens):
+            a = int(score_lens[b])
+            want_o = orc.gqa_attention(q[b:b + 1].float(), ks[b].float(), vs[b].float())[0, :, 0]
+            assert (out[b].cpu().float() - want_o).abs().max() < 2e-2, (sel, b)
+            want_s = orc.score_tokens(q[b:b + 1].float(), ks[b].float(), a, sel)[0]
+            assert float((scores[b, :a].cpu() - want_s).abs().max() / want_s.abs().max()) < 1e-4
+            # the same request stored contiguously: same tiles, same order of additions
+            o1, s1 = ops.dense_attn(q[b:b + 1].to(DEV), ks[b].to(DEV), vs[b].to(DEV), selector=sel, score_len=a)
+            op, sp = ops.dense_attn(q[b:b + 1].to(DEV), ops.PagedKV(kv.pool_k, kv.pool_v, kv.page_table[b:b + 1].contiguous(),
+                                                                      page_size), seq_len=n, selector=sel, score_len=a)
+            assert torch.equal(op, o1) and torch.equal(sp, s1), (sel, b)
+
+
+def test_ragged_topk_pads_with_minus_one_by_default():
+    """ops.topk without `out` on a ragged batch: entries beyond a request's own k are -1, which
+    is what PagedKV.slot_index treats as padding."""
+    g = torch.Generator().manual_seed(12)
+    lens = torch.tensor([900, 40, 20000], dtype=torch.int32)
+    ks = torch.tensor([60, 2, 1340], dtype=torch.int32)
+    s = torch.randn((3, int(lens.max())), generator=g)
+    idx = ops.topk(s.to(DEV), int(ks.max()), seq_lens=lens.to(DEV), k_per_seg=ks.to(DEV))
+    for b in range(3):
+        kb = int(ks[b])
+        assert torch.equal(idx[b, :kb].cpu().long(), orc.select_topk_stable(s[b:b + 1, : int(lens[b])], kb)[0])
+        assert (idx[b, kb:] == -1).all()
+    table, total = synth.shuffled_page_table(lens, 16)
+    pool = torch.zeros((total, 16, HKV, D), dtype=torch.bfloat16, device=DEV)
+    slots = ops.PagedKV(pool, pool, table.to(DEV), 16).slot_index(idx)
+    assert ((slots < 0) == (idx < 0)).all() and int(slots.max()) < total * 16
+
+
 def test_paged_gather_rows():
     lens = torch.tensor([300, 90], dtype=torch.int32)
     q, ks, vs, pool_k, pool_v, table = _paged_batch(lens, 16, torch.bfloat16, seed=4)

@@ -249,3 +249,30 @@ def test_filter_layer_suggestion_follows_the_cache_schedule():
         blob = trace.read_idx_tracer(tr.save_idx())
         assert blob["out"] == ["text"] and blob["layers_idx"][0][7][0]["prefill_len"] == 10
         assert torch.equal(blob["layers_idx"][0][7][0]["idx"], torch.tensor([[3, 1]]))
+
+
+def test_static_decode_budget_is_counted_on_the_host():
+    """Static (graph) decode appends at device positions nothing on the device checks: the
+    host counts the steps and refuses the one that would run past the buffers."""
+    from omnikv_amd.model import StaticDecodeGraph
+
+    c = okv_cache.OmniKVMultiStageCache([0, 1, 3], 3, 1, real_offload=False, max_new_tokens=4)
+    c._static_budget, c._static_steps = 3, 0
+    assert c.static_steps_left == 3
+
+    class FakeGraph:
+        replays = 0
+
+        def replay(self):
+            self.replays += 1
+
+    g = StaticDecodeGraph(FakeGraph(), c)
+    c.note_static_step()  # an eager static step
+    g.replay()
+    g.replay()
+    assert c.static_steps_left == 0 and g.graph.replays == 2
+    with pytest.raises(RuntimeError, match="max_new_tokens"):
+        g.replay()
+    assert g.graph.replays == 2  # the refused replay launched nothing
+    with pytest.raises(RuntimeError):
+        c.note_static_step()

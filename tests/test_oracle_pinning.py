@@ -273,3 +273,47 @@ def test_idx_overlap_score_against_python_sets():
     assert orc.idx_overlap_score(a, a + 20) == 0.0
     assert orc.idx_overlap_score(torch.arange(0, 10), torch.arange(0, 40)) == 1.0   # new inside old
     assert orc.idx_overlap_score(torch.arange(0, 40), torch.arange(0, 10)) == 0.25  # old inside new
+
+
+# ------------------------------------------------------------------ helpers for long contexts and pools
+@pytest.mark.parametrize("sel", ["last", "softmax_before_last", "softmax_sum_last"])
+def test_per_kv_head_evaluation_equals_the_whole_tensor_functions(sel):
+    g = torch.Generator().manual_seed(31)
+    q = torch.randn((2, 32, 1, 128), generator=g)
+    k = torch.randn((2, 8, 300, 128), generator=g)
+    v = torch.randn((2, 8, 300, 128), generator=g)
+    whole = orc.score_tokens(q, k, 257, sel)
+    by_head = orc.score_tokens_by_kv_head(q, k, 257, sel)
+    # the BLAS call sees other shapes, so sums may round differently: equal to fp32 rounding
+    assert torch.allclose(by_head, whole, rtol=2e-5, atol=2e-5 * float(whole.abs().max()))
+    assert torch.allclose(orc.gqa_attention_by_kv_head(q, k, v), orc.gqa_attention(q, k, v), rtol=1e-5, atol=1e-6)
+
+
+def test_paged_rows_round_trip_with_loops():
+    """Scatter a request into a shuffled pool token by token with Python loops; paged_rows
+    must read back exactly the original rows, for page sizes 1 (token slots), 4 and 16."""
+    g = torch.Generator().manual_seed(32)
+    for page_size, n in ((1, 9), (4, 10), (16, 33)):
+        pages = (n + page_size - 1) // page_size
+        table = torch.randperm(pages + 3, generator=g)[:pages]  # some pool pages stay unused
+        rows = torch.randn((1, 2, n, 8), generator=g)
+        pool = torch.full((pages + 3, page_size, 2, 8), float("nan"))
+        for t in range(n):
+            for h in range(2):
+                pool[int(table[t // page_size]), t % page_size, h] = rows[0, h, t]
+        assert torch.equal(orc.paged_rows(pool, table, n, page_size), rows)
+        assert torch.equal(orc.paged_rows(pool, table, n - 1, page_size), rows[:, :, : n - 1])
+
+
+def test_lightllm_raw_score_is_the_last_score_times_sqrt_d():
+    """The serving stack's score is the dot product before sm_scale: sqrt(D) times the `last`
+    selector's value (D = 64 makes the factor a power of two, so the identity is exact), and
+    against explicit loops."""
+    g = torch.Generator().manual_seed(33)
+    q = torch.randn((1, 8, 1, 64), generator=g)
+    k = torch.randn((1, 2, 50, 64), generator=g)
+    got = orc.lightllm_raw_head_max_score(q, k)
+    assert torch.equal(got, orc.score_tokens(q, k, 50, "last") * 8.0)
+    q64, k64 = q.double(), k.double()
+    want = [max(float((q64[0, h, 0] * k64[0, h // 4, t]).sum()) for h in range(8)) for t in range(50)]
+    assert torch.allclose(got[0].double(), torch.tensor(want, dtype=torch.float64), atol=1e-4)
