@@ -87,7 +87,7 @@ def _run_decode(dtype, real_offload, offload_mode, n=777, steps=3, L=8, sel_laye
             dk, dv = dut.update(k.to(DEV), v.to(DEV), i)
             assert torch.equal(dk.cpu(), rk) and torch.equal(dv.cpu(), rv)
         else:
-            prompt.append((k, v) if adopt == "lists_cpu" else (k.to(DEV), v.to(DEV)))
+            prompt.append((k.clone(), v.clone()) if adopt == "lists_cpu" else (k.to(DEV), v.to(DEV)))
     if adopt is not None:
         if adopt == "layers":
             src = _Bag(layers=[_Bag(keys=k, values=v) for k, v in prompt])
