@@ -210,6 +210,29 @@ int okv_sparse_attn(const void* q, const void* k_base, const void* v_base,
                     okv_stream_t stream);
 
 /*
+ * okv_sparse_attn without a workspace argument and without any allocation, for callers
+ * that can do neither: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  No counterpart in the reference.  Same arguments, same kernels and
+ * bit-identical output; the per-(q head, split) partial results go to a fixed array inside
+ * the library (okv_noalloc_scratch_bytes() = 4 MiB, held once per GPU the library runs on
+ * until the process ends).  Shapes whose okv_workspace_bytes(OKV_OP_SPARSE_ATTN, ...)
+ * exceed that return OKV_ERR_WORKSPACE (batch 1 fits up to several 100 000 selected rows, batch
+ * 16 several 10 000 per request).  The array is looked up once per device on the first
+ * call made with that device current -- make that first call outside a stream capture.
+ * Nothing in it needs clearing between calls (every partial that is read was written by
+ * the same call), but all calls on one GPU share it: calls that overlap in time on
+ * different streams of one GPU race.
+ */
+int okv_sparse_attn_noalloc(const void* q, const void* k_base, const void* v_base,
+                            const okv_kv_layout_t* layout, const int32_t* idx,
+                            int64_t idx_stride, const int32_t* sel_lens, int32_t max_sel_len,
+                            const void* tail_k, const void* tail_v, int64_t tail_token_stride,
+                            int64_t tail_head_stride, int64_t tail_batch_stride,
+                            const int32_t* tail_lens, int32_t max_tail_len, int32_t batch,
+                            float scale, void* out, okv_stream_t stream);
+int64_t okv_noalloc_scratch_bytes(void);
+
+/*
  * Materialised gather: dst[b][j][g][:] = src[b][idx[b][j]][g][:] for j < sel_len_b,
  * dst addressed by (dst_token_stride, dst_head_stride, dst_batch_stride).
  * Replaces torch.index_select(cache, 2, idx) in set_idx_on_gpu

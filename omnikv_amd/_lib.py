@@ -28,6 +28,8 @@ EXPORTS = (
     "okv_topk",
     "okv_dense_attn",
     "okv_sparse_attn",
+    "okv_sparse_attn_noalloc",
+    "okv_noalloc_scratch_bytes",
     "okv_gather_rows",
     "okv_offload_stage",
 )
@@ -91,6 +93,10 @@ def _declare(l):
     l.okv_dense_attn.argtypes = [vp, vp, vp, C.POINTER(KVLayout), vp, i32, i32, f32, vp, vp, i32, i32, i32, vp, i64, vp, sz, vp]
     l.okv_sparse_attn.restype = C.c_int
     l.okv_sparse_attn.argtypes = [vp, vp, vp, C.POINTER(KVLayout), vp, i64, vp, i32, vp, vp, i64, i64, i64, vp, i32, i32, f32, vp, vp, sz, vp]
+    l.okv_sparse_attn_noalloc.restype = C.c_int
+    l.okv_sparse_attn_noalloc.argtypes = l.okv_sparse_attn.argtypes[:-3] + [vp]
+    l.okv_noalloc_scratch_bytes.restype = C.c_int64
+    l.okv_noalloc_scratch_bytes.argtypes = []
     l.okv_gather_rows.restype = C.c_int
     l.okv_gather_rows.argtypes = [vp, C.POINTER(KVLayout), vp, i64, vp, i32, i32, vp, i64, i64, i64, vp]
     l.okv_offload_stage.restype = C.c_int

@@ -10,6 +10,8 @@
 #include <math.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "okv_internal.h"
 #include "okv_device.h"
 
@@ -579,5 +581,57 @@ int okv_sparse_attn(const void* q, const void* k_base, const void* v_base,
   return launch_attention(q, r, layout, batch, scale, out, true, 0, 0, nullptr, 0, w,
                           (hipStream_t)stream);
 }
+
+// ---------------------------------------------------------------------------
+// Sparse attention for callers that can neither allocate nor bring a workspace: the
+// per-(q head, split) partials live in a fixed array of the library's own, one copy per
+// GPU.  Host code never passes the array's name to a kernel (on the host it is only a
+// stand-in): the device address is asked for once per device and used from then on.
+constexpr size_t kScratchBytes = (size_t)4 << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kMaxScratchDevices = 64;
+static void* g_scratch_ptr[kMaxScratchDevices];  // [device] -> that GPU's copy of `scratch`
+static std::mutex g_scratch_mutex;
+
+static int scratch_of_current_device(void** out) {
+  int dev = -1;
+  OKV_HIP_CHECK(hipGetDevice(&dev));
+  OKV_REQUIRE(dev >= 0 && dev < kMaxScratchDevices, OKV_ERR_UNSUPPORTED, "device %d: at most %d devices", dev,
+              kMaxScratchDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    OKV_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    OKV_REQUIRE(p != nullptr, OKV_ERR_HIP, "hipGetSymbolAddress returned a NULL address");
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return OKV_OK;
+}
+
+int okv_sparse_attn_noalloc(const void* q, const void* k_base, const void* v_base,
+                            const okv_kv_layout_t* layout, const int32_t* idx, int64_t idx_stride,
+                            const int32_t* sel_lens, int32_t max_sel_len, const void* tail_k,
+                            const void* tail_v, int64_t tail_token_stride, int64_t tail_head_stride,
+                            int64_t tail_batch_stride, const int32_t* tail_lens, int32_t max_tail_len,
+                            int32_t batch, float scale, void* out, okv_stream_t stream) {
+  OKV_REQUIRE(layout != nullptr, OKV_ERR_INVALID, "layout is NULL");
+  OKV_REQUIRE(batch >= 1 && max_sel_len >= 0 && max_tail_len >= 0, OKV_ERR_INVALID, "bad batch or length");
+  const size_t need = attn_workspace_bytes(batch, layout->num_q_heads, layout->num_kv_heads, layout->head_dim,
+                                           max_sel_len, max_tail_len, 0, true, false, nullptr, nullptr, true);
+  OKV_REQUIRE(need <= kScratchBytes, OKV_ERR_WORKSPACE,
+              "okv_sparse_attn_noalloc: batch %d x (%d selected + %d tail) rows needs %zu bytes of partial "
+              "results, the library's fixed scratch holds %zu; use okv_sparse_attn with a workspace",
+              batch, max_sel_len, max_tail_len, need, kScratchBytes);
+  void* ws = nullptr;
+  int rc = scratch_of_current_device(&ws);
+  if (rc) return rc;
+  // every partial the merge reads is written by the split pass of the same call: nothing to clear
+  return okv_sparse_attn(q, k_base, v_base, layout, idx, idx_stride, sel_lens, max_sel_len, tail_k, tail_v,
+                         tail_token_stride, tail_head_stride, tail_batch_stride, tail_lens, max_tail_len, batch,
+                         scale, out, ws, kScratchBytes, stream);
+}
+
+int64_t okv_noalloc_scratch_bytes(void) { return (int64_t)kScratchBytes; }
 
 }  // extern "C"
