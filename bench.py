@@ -11,8 +11,12 @@ layers 0-1, sparse attention over the selected rows + tail everywhere else.
 One step = the attention work of one decode step over all 32 layers.
 
 Prints ONE JSON line: metric = microseconds of attention per layer (step time /
-32), plus `roofline` for the dominant kernel (dense split attention) and
-`cpu_baseline` (the CPU oracle timed on this host on a bounded sample).
+32); `roofline` for the dominant kernel (dense split attention); `roofline_by_kernel`
+for every kernel of the step (scoring, filter pass, sparse gather-attention, top-k, and
+the load-only floor of the sparse layer), each timed live with events around a replayed
+graph of that kernel alone; `variants` (the reference's `last` selector; k = round
+instead of floor); `cpu_baseline` (the CPU oracle at this context on a bounded sample)
+and `cpu_baseline_config0` (the CPU-runnable 4096-token configuration).
 """
 from __future__ import annotations
 
@@ -108,17 +112,6 @@ def make_step(ks, vs, qs, n, tail, k_sel, selector):
     return step
 
 
-def time_events(fn, reps, stream):
-    """Average milliseconds of fn() between two events on `stream`."""
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for _ in range(reps):
-        fn()
-    e1.record(stream)
-    e1.synchronize()
-    return e0.elapsed_time(e1) / reps
-
-
 def cpu_baseline(n, k_sel, selector, budget_s=25.0):
     """The CPU oracle on this host: one dense layer, one filter layer (score +
     top-k + dense attention) and one sparse layer (gather + cat + attention) at
@@ -170,6 +163,167 @@ def cpu_baseline(n, k_sel, selector, budget_s=25.0):
     }
 
 
+def time_graph(fn, launches, reps, stream):
+    """Microseconds per launch of fn()'s `launches` launches: captured once, replayed between two events."""
+    fn()
+    stream.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=stream):
+        fn()
+    g.replay()
+    stream.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(reps):
+        g.replay()
+    e1.record(stream)
+    e1.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (reps * launches)
+
+
+def measure_kernels(ops, l, check, stream, ks, vs, qs, n, tail, k_sel, selector, dtype, esize, dense_layers,
+                    sparse_layers, filter_layers, idx):
+    """Per-kernel microseconds and fraction of the HBM roofline (algorithmic bytes / time / 8 TB/s) for the
+    kernels the decode step is made of.  `..._split_pass` entries time the split pass alone (the library's
+    measurement hook suppresses the merge / finishing launch), `..._op` entries the whole entry point."""
+    import ctypes as C
+
+    from omnikv_amd import _lib
+
+    reps = 20
+    kv_row = HKV * D * esize
+    tname = {torch.bfloat16: "BF16", torch.float16: "F16", torch.float32: "float"}[dtype]
+    mfma = dtype != torch.float32
+    out = {}
+
+    def entry(name, kernel, us, nbytes, launches_per_op=1, note=None):
+        e = {"kernel": kernel, "us": us, "launches": launches_per_op}
+        if nbytes:
+            e.update({"bytes": nbytes, "achieved": nbytes / (us * 1e-6) / 1e9, "frac": nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                      "bound": "hbm", "unit": "GB/s"})
+        else:
+            e.update({"bound": "latency"})
+        if note:
+            e["note"] = note
+        out[name] = e
+
+    def full(layer):
+        return ks[layer][:, :, : n + tail], vs[layer][:, :, : n + tail]
+
+    def split_only(fn, launches):
+        check(l.okv_diag_split_pass_only(1))
+        try:
+            return time_graph(fn, launches, reps, stream)
+        finally:
+            check(l.okv_diag_split_pass_only(0))
+
+    def dense():
+        for layer in dense_layers:
+            ops.dense_attn(qs[layer], *full(layer))
+
+    dense_bytes = 2.0 * (n + tail) * kv_row
+    stage1 = "okv::attn_stage1_mfma<%s,4,%%s,%%d,%%s>" % tname if mfma else "okv::attn_stage1_generic<float,4,%s> [mode %d, logits %s]"
+    entry("dense_split_pass", stage1 % ("true", 0, "false") + " (dense split pass over N+tail rows of K and V)",
+          split_only(dense, len(dense_layers)), dense_bytes)
+    entry("dense_attention_op", "split pass + okv::attn_merge", time_graph(dense, len(dense_layers), reps, stream), dense_bytes, 2)
+
+    def fused():
+        for layer in filter_layers:
+            ops.dense_attn(qs[layer], *full(layer), selector=selector, score_len=n)
+
+    fused_bytes = dense_bytes + 4.0 * n
+    entry("filter_layer_split_pass", stage1 % ("true", 0, "true") + f" (attention + {selector} logits in one pass over K)",
+          split_only(fused, len(filter_layers)), fused_bytes)
+    entry("filter_layer_op", "split pass + okv::merge_and_finish", time_graph(fused, len(filter_layers), reps, stream),
+          fused_bytes, 2)
+
+    score_bytes = 1.0 * n * kv_row + 4.0 * n
+
+    def score_last():
+        for layer in filter_layers:
+            ops.score(qs[layer], ks[layer][:, :, :n], selector="last")
+
+    entry("score_last_op", "okv::score_raw_mfma<%s,4,false> (raw logits, head max: one launch)" % tname if mfma
+          else "split pass + finish", time_graph(score_last, len(filter_layers), reps, stream), score_bytes, 1 if mfma else 2)
+
+    def score_soft():
+        for layer in filter_layers:
+            ops.score(qs[layer], ks[layer][:, :, :n], selector="softmax_sum_last")
+
+    entry("score_softmax_split_pass", stage1 % ("false", 0, "true") + " (softmax_sum_last: logits + per-split log-sum-exp)",
+          split_only(score_soft, len(filter_layers)), score_bytes)
+    entry("score_softmax_op", "split pass + okv::merge_and_finish", time_graph(score_soft, len(filter_layers), reps, stream),
+          score_bytes, 2)
+
+    any_idx = next(iter(idx.values()))
+    sc = ops.score(qs[filter_layers[0]], ks[filter_layers[0]][:, :, :n], selector=selector)
+    entry("topk_op", "okv::topk_mb_hist + topk_mb_cand + topk_mb_write (k = %d of %d)" % (k_sel, n),
+          time_graph(lambda: [ops.topk(sc, k_sel) for _ in range(4)], 4, reps, stream), None, 3)
+
+    def sparse():
+        for layer in sparse_layers:
+            ops.sparse_attn(qs[layer], ks[layer][:, :, :n], vs[layer][:, :, :n], idx=any_idx,
+                            tail_k=ks[layer][:, :, n: n + tail], tail_v=vs[layer][:, :, n: n + tail])
+
+    sparse_bytes = 2.0 * (k_sel + tail) * kv_row + 4.0 * k_sel
+    entry("sparse_split_pass", stage1 % ("true", 1, "false") + " (fused gather + attention over the selected rows + tail)",
+          split_only(sparse, len(sparse_layers)), sparse_bytes)
+    entry("sparse_attention_op", "split pass + okv::attn_merge", time_graph(sparse, len(sparse_layers), reps, stream),
+          sparse_bytes, 2)
+    if mfma:
+        # the attainable bound on this device: a kernel with the same grid, index lookups, load shapes and
+        # bytes that does nothing with what it loads
+        shape = _lib.Shape(1, HQ, HKV, D, k_sel, tail, 0)
+        rows_, splits_ = C.c_int32(0), C.c_int32(0)
+        check(l.okv_diag_split_geometry(_lib.OKV_OP_SPARSE_ATTN, C.byref(shape), C.byref(rows_), C.byref(splits_)))
+        sink = torch.zeros(4, dtype=torch.int32, device=any_idx.device)
+        k0 = ks[sparse_layers[0]]
+        lay = _lib.KVLayout(_lib.OKV_BF16 if dtype == torch.bfloat16 else _lib.OKV_F16, HQ, HKV, D, k0.stride(2),
+                            k0.stride(1), k0.stride(0), None, 0, 0, 0)
+
+        def floor():
+            for layer in sparse_layers:
+                check(l.okv_diag_gather_floor(ks[layer].data_ptr(), vs[layer].data_ptr(), C.byref(lay), any_idx.data_ptr(),
+                                              k_sel, rows_.value, sink.data_ptr(), stream.cuda_stream))
+
+        entry("sparse_load_only_floor", "okv::gather_floor_kernel (same grid, index lookups and loads; no arithmetic, no output)",
+              time_graph(floor, len(sparse_layers), reps, stream), 2.0 * k_sel * kv_row + 4.0 * k_sel,
+              note="split_rows %d, %d splits x %d kv heads" % (rows_.value, (k_sel + rows_.value - 1) // rows_.value, HKV))
+
+        def empty():
+            for _ in range(24):
+                check(l.okv_diag_empty_launch(sink.data_ptr(), stream.cuda_stream))
+
+        entry("empty_launch", "okv::empty_kernel (one wave, no work): the cost of a launch inside a replayed graph",
+              time_graph(empty, 24, reps, stream), None)
+    return out
+
+
+def cpu_baseline_config0(n=4096, ratio=0.067):
+    """The CPU-runnable configuration itself (batch 1, fp32, 4096 tokens): the oracle's whole filter-layer op
+    -- score, top-k, gather, one downstream layer's attention over the selected rows -- for both selectors."""
+    from omnikv_amd import synth
+    from oracle import okv_oracle as orc
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    q, k, v = synth.filter_layer_inputs(n, HQ, HKV, D)
+    _, k2, v2 = synth.filter_layer_inputs(n, HQ, HKV, D, seed=synth.SEED_DATA + 100)
+    qn = synth.fresh_q()
+    res = {"context": n, "dtype": "f32", "cores": cores, "kind": "port", "unit": "us per filter-layer op",
+           "sample": "median of 20 runs after 3 warm-ups of okv_oracle.filter_layer_op (score + top-k + gather + sparse attention)"}
+    for sel in ("last", "softmax_sum_last"):
+        for kk in sorted({int(ratio * n), int(round(ratio * n))}):
+            ts = []
+            for i in range(23):
+                t0 = time.perf_counter()
+                orc.filter_layer_op(q, k, v2, k2, qn, kk, sel)
+                ts.append(time.perf_counter() - t0)
+            ts = sorted(ts[3:])
+            res[f"{sel}_k{kk}"] = ts[len(ts) // 2] * 1e6
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -185,7 +339,7 @@ def main():
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32"])
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--detail", action="store_true", help="print per-op timings to stderr")
+    ap.add_argument("--no-variants", action="store_true", help="skip the extra steps (selector last, k = round(ratio N))")
     ap.add_argument("--split-rows", type=int, default=0, help="override rows per split (0 = automatic)")
     ap.add_argument("--attn-variant", type=int, default=0, help="1 = portable VALU stage 1 for every dtype")
     args = ap.parse_args()
@@ -249,52 +403,46 @@ def main():
         def pct(p):
             return per_step[min(len(per_step) - 1, int(p * len(per_step)))]
 
-        # ---- dominant kernel: dense split attention over N+tail rows, eager, events
-        dense_layers = [l for l, kd in schedule().items() if kd[0] == "dense"]
-        reps = 10
+        # ---- single kernels, timed live: each measurement captures one pass over its layers in a HIP
+        # graph (so short kernels are not paced by the host's launch rate) and replays it between two
+        # events on this stream; the layers rotate, so no launch finds its rows in cache
+        kinds = schedule()
+        dense_layers = [l for l, kd in kinds.items() if kd[0] == "dense"]
+        sparse_layers = [l for l, kd in kinds.items() if kd[0] == "sparse"]
+        fl = list(FILTER_LAYERS)
+        by_kernel = measure_kernels(ops, lib(), check, stream, ks, vs, qs, n, tail, k_sel, args.selector, dtype, esize,
+                                    dense_layers, sparse_layers, fl, idx)
+        dom = by_kernel["dense_split_pass"]
+        split_us, dense_us = dom["us"], by_kernel["dense_attention_op"]["us"]
 
-        def dense_pass():
-            for l in dense_layers:
-                ops.dense_attn(qs[l], ks[l][:, :, : n + tail], vs[l][:, :, : n + tail])
-
-        dense_pass()
-        dense_ms = time_events(dense_pass, reps, stream) / len(dense_layers)
-        # the split pass alone (the dominant kernel), merge launch left out
-        check(lib().okv_set_option(b"skip_merge", 1))
-        dense_pass()
-        split_ms = time_events(dense_pass, reps, stream) / len(dense_layers)
-        check(lib().okv_set_option(b"skip_merge", 0))
-        detail = {}
-        if args.detail:
-            fl = FILTER_LAYERS[0]
-            sp = [l for l, kd in schedule().items() if kd[0] == "sparse"]
-            _, sc = ops.dense_attn(qs[fl], ks[fl][:, :, : n + tail], vs[fl][:, :, : n + tail],
-                                   selector=args.selector, score_len=n)
-            ix = ops.topk(sc, k_sel)
-            detail["fused_filter_ms"] = time_events(
-                lambda: [ops.dense_attn(qs[l], ks[l][:, :, : n + tail], vs[l][:, :, : n + tail],
-                                        selector=args.selector, score_len=n) for l in FILTER_LAYERS], reps, stream) / 3
-            detail["score_only_ms"] = time_events(
-                lambda: [ops.score(qs[l], ks[l][:, :, :n], selector=args.selector) for l in FILTER_LAYERS], reps, stream) / 3
-            detail["score_raw_max_ms"] = time_events(
-                lambda: [ops.score(qs[l], ks[l][:, :, :n], selector="last") for l in FILTER_LAYERS], reps, stream) / 3
-            detail["topk_ms"] = time_events(lambda: ops.topk(sc, k_sel), 20, stream)
-            detail["sparse_ms"] = time_events(
-                lambda: [ops.sparse_attn(qs[l], ks[l][:, :, :n], vs[l][:, :, :n], idx=ix,
-                                         tail_k=ks[l][:, :, n: n + tail], tail_v=vs[l][:, :, n: n + tail]) for l in sp],
-                reps, stream) / len(sp)
-            detail["dense_ms"] = dense_ms
-            print(json.dumps(detail), file=sys.stderr)
+        # ---- the same step with the reference's own selector and with BASELINE's k = round(0.067 N)
+        variants = {}
+        if not args.no_variants:
+            for name, sel_v, k_v in (("selector_last", "last", k_sel), ("selected_%d" % round(args.ratio * n), args.selector,
+                                                                         int(round(args.ratio * n)))):
+                step_v = make_step(ks, vs, qs, n, tail, k_v, sel_v)
+                step_v()
+                stream.synchronize()
+                gv = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gv, stream=stream):
+                    step_v()
+                gv.replay()
+                stream.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(args.steps):
+                    gv.replay()
+                stream.synchronize()
+                ms = (time.perf_counter() - t0) * 1e3 / args.steps
+                variants[name] = {"selector": sel_v, "selected": k_v, "ms_per_step": ms, "us_per_layer": ms * 1e3 / LAYERS}
 
     dense_bytes = 2.0 * (n + tail) * HKV * D * esize  # K and V rows once each
-    achieved = dense_bytes / (split_ms * 1e-3) / 1e9
-    kinds = schedule()
     step_bytes = 0.0
     for l, (kind, _) in kinds.items():
         if kind in ("dense", "filter"):
             step_bytes += dense_bytes + (4.0 * n if kind == "filter" else 0.0)
         else:
             step_bytes += 2.0 * (k_sel + tail) * HKV * D * esize + 4.0 * k_sel
+    traffic = TRAFFIC_BYTES.get((n, tail, args.dtype))
     res = {
         "metric": "omnikv_decode_step_attn_us_per_layer",
         "value": wall_ms * 1e3 / LAYERS,
@@ -320,16 +468,20 @@ def main():
         "step_hbm_gbs": step_bytes / (wall_ms * 1e-3) / 1e9,
         "step_ms_p10_p50_p90": [round(pct(0.1), 4), round(pct(0.5), 4), round(pct(0.9), 4)],
         "roofline": {
-            "kernel": "okv::attn_stage1_mfma<BF16,4,true,0,false> (dense split pass over N+tail rows of K and V)"
-            if dtype != torch.float32 else "okv::attn_stage1_generic<float,4,true> (dense split pass)",
-            "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES.get((n, tail, args.dtype)),
-            "bytes_per_launch": dense_bytes, "avg_launch_us": split_ms * 1e3,
-            "with_merge_launch_us": dense_ms * 1e3,
+            "kernel": dom["kernel"],
+            "bound": "hbm", "achieved": dom["achieved"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": dom["frac"], "traffic": traffic,
+            "traffic_source": "profiles/dense_split_pass_pmc.txt (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of an earlier "
+                              "run of this kernel at this shape; not measured in this run)" if traffic else None,
+            "bytes_per_launch": dense_bytes, "avg_launch_us": split_us,
+            "with_merge_launch_us": dense_us,
         },
+        "roofline_by_kernel": by_kernel,
+        "variants": variants,
     }
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(n, k_sel, args.selector)
+        res["cpu_baseline_config0"] = cpu_baseline_config0()
     print(json.dumps(res))
 
 

@@ -17,7 +17,8 @@
  *   - return value: 0 on success, a negative okv_status otherwise; the library
  *     never throws and never aborts; okv_strerror() names a code and
  *     okv_last_error() gives the detail of the calling thread's last failure;
- *   - calls on different streams may run concurrently if their workspaces differ.
+ *   - calls on different streams, from one or several host threads, may run concurrently
+ *     if their workspaces differ (okv_set_option is the exception, see there).
  *
  * Tensors
  *   q, out     (batch, num_q_heads, head_dim) contiguous, same dtype as K/V
@@ -99,9 +100,10 @@ int okv_version(void);
 /* Process-wide tuning switches, for A/B measurements.  "attn_variant": 0 (default)
  * runs 16-bit attention / scoring on the matrix-core kernel, 1 forces the portable
  * VALU kernel for every dtype.  "split_rows": rows per split of the attention /
- * scoring pass, 0 = automatic.  "skip_merge": 1 launches the split pass of the
- * attention entry points alone (outputs are then NOT produced; for timing that kernel
- * in isolation).  Set options before sizing workspaces.  No reference counterpart. */
+ * scoring pass (a multiple of 16), 0 = automatic.  An option applies to every later
+ * call of every thread and changes workspace sizes: set options before sizing
+ * workspaces and before other threads call into the library, not while they do.
+ * No reference counterpart. */
 int okv_set_option(const char* name, int value);
 
 /* Bytes of scratch `op` needs for `shape`.  No reference counterpart: the

@@ -82,6 +82,14 @@ def _declare(l):
     l.okv_workspace_bytes.argtypes = [C.c_int, C.POINTER(Shape), C.POINTER(sz)]
     l.okv_set_option.restype = C.c_int
     l.okv_set_option.argtypes = [C.c_char_p, C.c_int]
+    l.okv_diag_split_pass_only.restype = C.c_int  # measurement hook, not part of the public header
+    l.okv_diag_split_pass_only.argtypes = [C.c_int]
+    l.okv_diag_split_geometry.restype = C.c_int
+    l.okv_diag_split_geometry.argtypes = [C.c_int, C.POINTER(Shape), C.POINTER(i32), C.POINTER(i32)]
+    l.okv_diag_gather_floor.restype = C.c_int
+    l.okv_diag_gather_floor.argtypes = [vp, vp, C.POINTER(KVLayout), vp, i32, i32, vp, vp]
+    l.okv_diag_empty_launch.restype = C.c_int
+    l.okv_diag_empty_launch.argtypes = [vp, vp]
     l.okv_score.restype = C.c_int
     l.okv_score.argtypes = [vp, vp, C.POINTER(KVLayout), vp, i32, i32, i32, i32, f32, vp, i64, vp, sz, vp]
     l.okv_score_window.restype = C.c_int

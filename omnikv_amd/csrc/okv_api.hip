@@ -19,7 +19,7 @@ static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; 
 
 // Rows per split: enough blocks to fill 256 CUs several times over for long
 // contexts, never below one 64-row tile group.
-int g_split_rows_override = 0;
+std::atomic<int> g_split_rows_override{0};
 
 static int num_compute_units() {
   static int cus = 0;
@@ -42,7 +42,8 @@ static int num_compute_units() {
 // 53.1 sized for six).  The cap keeps the LDS staging of a scored split's logits small.
 static int choose_split_rows(int batch, int hq, int hkv, int total_rows, bool with_v,
                              bool with_logits, bool gather) {
-  if (g_split_rows_override > 0) return g_split_rows_override;
+  const int forced = g_split_rows_override.load(std::memory_order_relaxed);
+  if (forced > 0) return forced;
   (void)gather;
   // a batch is sized by its longest request, so ragged ones fill less than the grid suggests:
   // three and six per CU there (measured on 16 requests of 8K..32K tokens)

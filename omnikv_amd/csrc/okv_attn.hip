@@ -10,6 +10,7 @@
 #include <math.h>
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "okv_internal.h"
@@ -345,8 +346,8 @@ __global__ __launch_bounds__(256) void merge_and_finish(RowList rows, int hq, At
 }
 
 // ----------------------------------------------------------------- launch
-int g_attn_variant = 0;  // 0 = pick per dtype, 1 = portable VALU stage 1 everywhere
-int g_skip_merge = 0;    // 1 = launch the split pass alone (timing it in isolation)
+std::atomic<int> g_attn_variant{0};  // 0 = pick per dtype, 1 = portable VALU stage 1 everywhere
+std::atomic<int> g_split_pass_only{0};  // diagnostic (okv_diag_split_pass_only): no merge / finish launch
 
 bool launch_stage1_mfma(int dtype, const void* q, const RowList& rows, int hq, int hkv, int batch,
                         float scale, const AttnWorkspace& w, bool with_v, bool write_logits,
@@ -376,7 +377,7 @@ static int launch_typed(const void* q, const RowList& rows, const okv_kv_layout_
   const int hq = lay->num_q_heads, hkv = lay->num_kv_heads, G = hq / hkv;
   const bool want_scores = scores != nullptr;
   // raw scores alone need no normaliser: one launch that reduces the heads in the workgroup
-  if (g_attn_variant != 1 && !with_v && want_scores && normalise == OKV_NORM_RAW &&
+  if (g_attn_variant.load(std::memory_order_relaxed) != 1 && !with_v && want_scores && normalise == OKV_NORM_RAW &&
       launch_score_raw_mfma(lay->dtype, q, rows, hq, hkv, batch, scale, head_reduce, scores, score_stride,
                             stream)) {
     OKV_HIP_CHECK(hipGetLastError());
@@ -388,7 +389,7 @@ static int launch_typed(const void* q, const RowList& rows, const okv_kv_layout_
     wm.logit_heads = hkv;
   }
   const AttnWorkspace* used = &w;
-  if (g_attn_variant != 1 &&
+  if (g_attn_variant.load(std::memory_order_relaxed) != 1 &&
       launch_stage1_mfma(lay->dtype, q, rows, hq, hkv, batch, scale, wm, with_v, want_scores, stream)) {
     used = &wm;  // 16-bit K/V: stage 1 ran on the matrix-core kernel
   } else
@@ -401,13 +402,15 @@ static int launch_typed(const void* q, const RowList& rows, const okv_kv_layout_
   }
   const bool need_score_lse = want_scores && normalise == OKV_NORM_SOFTMAX;
   const int finish_blocks = want_scores ? (rows.max_score_len + 1023) / 1024 : 0;
-  if (!g_skip_merge && finish_blocks > 0 && hq <= kMaxFinishHeads) {
+  if (g_split_pass_only.load(std::memory_order_relaxed)) {
+    // measurement hook: the split pass alone
+  } else if (finish_blocks > 0 && hq <= kMaxFinishHeads) {
     // one launch: the merge of the outputs next to the finishing of the scores
     hipLaunchKernelGGL((merge_and_finish<T>), dim3((with_v ? hq : 0) + finish_blocks, batch), dim3(256), 0,
                        stream, rows, hq, *used, (T*)out, with_v ? hq : 0, head_reduce, normalise, scores,
                        score_stride);
   } else {
-    if (!g_skip_merge && (with_v || need_score_lse))
+    if (with_v || need_score_lse)
       hipLaunchKernelGGL((attn_merge<T>), dim3(hq, batch), dim3(256), 0, stream, rows, hq, *used,
                          (T*)out, (int)with_v, (int)need_score_lse);
     if (finish_blocks > 0)
@@ -460,19 +463,22 @@ int okv_set_option(const char* name, int value) {
     g_attn_variant = value;
     return OKV_OK;
   }
-  if (strcmp(name, "skip_merge") == 0) {
-    OKV_REQUIRE(value == 0 || value == 1, OKV_ERR_INVALID, "skip_merge must be 0 or 1");
-    g_skip_merge = value;
-    return OKV_OK;
-  }
   if (strcmp(name, "split_rows") == 0) {
-    OKV_REQUIRE(value == 0 || (value >= 64 && value <= 8192 && value % 64 == 0), OKV_ERR_INVALID,
-                "split_rows must be 0 (automatic) or a multiple of 64 in [64, 8192]");
+    OKV_REQUIRE(value == 0 || (value >= 64 && value <= 8192 && value % 16 == 0), OKV_ERR_INVALID,
+                "split_rows must be 0 (automatic) or a multiple of 16 in [64, 8192]");
     g_split_rows_override = value;
     return OKV_OK;
   }
   set_error("unknown option %s", name);
   return OKV_ERR_INVALID;
+}
+
+// Measurement hook, deliberately absent from the public header: with 1 the attention / scoring
+// entry points launch their split pass alone (outputs are then not produced), so that a timer
+// around the call measures that kernel.  Process-wide; never set it in a serving process.
+int okv_diag_split_pass_only(int on) {
+  g_split_pass_only.store(on ? 1 : 0, std::memory_order_relaxed);
+  return OKV_OK;
 }
 
 int okv_score(const void* q, const void* k_base, const okv_kv_layout_t* layout,

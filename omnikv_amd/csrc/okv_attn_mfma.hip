@@ -17,6 +17,8 @@
 // tile t is consumed.  The sixteen lane rows of the block meet in LDS at the end.
 #include <math.h>
 
+#include <atomic>
+
 #include "okv_device.h"
 #include "okv_internal.h"
 
@@ -399,11 +401,13 @@ static void launch_one(const void* q, const RowList& rows, int hq, int hkv, int 
   if (LOGITS && (size_t)G * w.split_rows > lds_floats) lds_floats = (size_t)G * w.split_rows;
   if (stage1_k_through_lds(MODE)) lds_floats += 4 * 1024;  // 4 KB of K staging per wave
   const size_t lds_bytes = lds_floats * sizeof(float);
-  static size_t configured = 0;
-  if (lds_bytes > configured) {
+  static std::atomic<size_t> configured{0};  // per instantiation; two threads raising it at once both succeed
+  if (lds_bytes > configured.load(std::memory_order_relaxed)) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    configured = lds_bytes;
+    size_t seen = configured.load(std::memory_order_relaxed);
+    while (seen < lds_bytes && !configured.compare_exchange_weak(seen, lds_bytes, std::memory_order_relaxed)) {
+    }
   }
   dim3 grid(hkv, w.max_splits, batch);  // kv head fastest: co-resident blocks cover whole token rows
   hipLaunchKernelGGL(kern, grid, dim3(256), lds_bytes, stream, (const T*)q, rows, hq, scale, w);

@@ -5,6 +5,8 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <atomic>
+
 #include "../../include/omnikv_hip.h"
 
 namespace okv {
@@ -148,7 +150,7 @@ int carve_attn_workspace(void* ws, size_t ws_bytes, int batch, int hq, int hkv, 
                          int max_main, int max_tail, int max_score, bool with_v,
                          bool with_logits, AttnWorkspace* out, bool gather = false);
 
-extern int g_split_rows_override;  // 0 = automatic
+extern std::atomic<int> g_split_rows_override;  // 0 = automatic
 
 int validate_layout(const okv_kv_layout_t* layout, const void* k_base, const void* v_base);
 

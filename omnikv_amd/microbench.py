@@ -24,7 +24,7 @@ HQ, HKV, D = 32, 8, 128
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--op", required=True,
-                    choices=["dense", "fused", "score", "topk", "sparse", "sparse_packed", "gather", "copy",
+                    choices=["dense", "fused", "score", "topk", "sparse", "sparse_packed", "sparse_floor", "empty", "gather", "copy",
                              "offload_memcpy", "offload_zero_copy", "h2d", "window", "window_loop",
                              "paged_dense", "paged_fused", "paged_score", "paged_topk", "paged_sparse", "paged_sparse_slots"])
     ap.add_argument("--batch", type=int, default=16, help="requests of the paged_* ops (ragged lengths 8192..32768)")
@@ -100,8 +100,28 @@ def main():
             hsrc = torch.empty(k_sel * 2 * HKV * D * es, dtype=torch.uint8).pin_memory()
             hdst = torch.empty(k_sel * 2 * HKV * D * es, dtype=torch.uint8, device=dev)
 
+    floor = None
+    if args.op in ("sparse_floor", "empty"):
+        # measurement kernels of the library: a load-only pass with the sparse layer's grid, index lookups,
+        # load shapes and bytes (what merely fetching the rows costs here), and an empty launch
+        import ctypes as C
+
+        from . import _lib
+        shape = _lib.Shape(1, HQ, HKV, D, k_sel, tail, 0)
+        rows_, splits_ = C.c_int32(0), C.c_int32(0)
+        check(lib().okv_diag_split_geometry(_lib.OKV_OP_SPARSE_ATTN, C.byref(shape), C.byref(rows_), C.byref(splits_)))
+        sink = torch.zeros(4, dtype=torch.int32, device=dev)
+        lay = _lib.KVLayout(ops._DTYPES[dtype], HQ, HKV, D, ks[0].stride(2), ks[0].stride(1), ks[0].stride(0), None, 0, 0, 0)
+        floor = (rows_.value, sink, lay, C)
+
     def call(i):
         l = i % nl
+        if args.op == "sparse_floor":
+            rows, sink, lay, C = floor
+            return check(lib().okv_diag_gather_floor(ks[l].data_ptr(), vs[l].data_ptr(), C.byref(lay), idx.data_ptr(), k_sel,
+                                                     rows, sink.data_ptr(), torch.cuda.current_stream().cuda_stream))
+        if args.op == "empty":
+            return check(lib().okv_diag_empty_launch(floor[1].data_ptr(), torch.cuda.current_stream().cuda_stream))
         if args.op == "dense":
             return ops.dense_attn(qs[l], ks[l], vs[l])
         if args.op == "fused":
@@ -147,6 +167,8 @@ def main():
         "window_loop": 1.0 * n * row + 4.0 * n,
         "sparse": 2.0 * (k_sel + tail) * row + 4.0 * k_sel,
         "sparse_packed": 2.0 * (k_sel + tail) * row,
+        "sparse_floor": 2.0 * k_sel * row + 4.0 * k_sel,
+        "empty": 0.0,
         "gather": 2.0 * k_sel * row + 4.0 * k_sel,
         "copy": 2.0 * (n + tail) * row,
         "h2d": 2.0 * k_sel * row,
