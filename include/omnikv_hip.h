@@ -263,6 +263,34 @@ int okv_offload_stage(const void* host_src, int64_t row_bytes, const int32_t* ho
                       int32_t n_rows, void* host_staging, int32_t host_threads,
                       void* dev_dst, okv_stream_t copy_stream, void* done_event);
 
+/*
+ * real_offload tier, incremental.  The rows staged on the device for a group of sparse
+ * layers are a set -- attention over them does not depend on their order -- so a new selection
+ * keeps the rows it shares with the previous one in place and fetches only the others, into
+ * the slots the dropped rows free.  okv_offload_plan (once per selection; one workgroup, all
+ * arrays in device memory) updates the two maps
+ *   slot_tok[k]          token whose row sits in slot s, -1 for an empty slot
+ *   slot_of[num_tokens]  slot of token t, -1 when it is not staged
+ * (both filled with -1 before the first selection) from idx_new[k] (ascending, distinct,
+ * < num_tokens) and writes the exchange: fetch_tok[r] -> slot fetch_slot[r] for
+ * r < fetch_count[0], tokens ascending, slots ascending.  k <= 262144.  okv_offload_fetch
+ * (once per layer of the group) then copies those rows: row fetch_tok[r] of src (rows of
+ * row_bytes bytes, a multiple of 16; pinned host memory that the device can read, or device
+ * memory) into row fetch_slot[r] of dev_dst.  max_rows (<= k) bounds the launch; the count
+ * itself is read on the device, so both calls can be captured in a HIP graph.  The staged
+ * buffer is then attended with okv_sparse_attn(idx = NULL, sel_len = k).
+ * Replaces the full re-copy `index_select(cpu cache, 2, idx.cpu()).cuda()` that
+ * set_idx_on_gpu repeats at every selection (modeling/spec_cache.py:293-303) and goes further
+ * than the lazy variant, which can only skip a selection as a whole
+ * (OmniKVLazyCache.set_out_idx, modeling/spec_cache.py:539-557).
+ */
+int okv_offload_plan(const int32_t* idx_new, int32_t k, int32_t* slot_tok, int32_t* slot_of,
+                     int32_t num_tokens, int32_t* fetch_tok, int32_t* fetch_slot,
+                     int32_t* fetch_count, okv_stream_t stream);
+int okv_offload_fetch(const void* src, int64_t row_bytes, const int32_t* fetch_tok,
+                      const int32_t* fetch_slot, const int32_t* fetch_count, int32_t max_rows,
+                      void* dev_dst, okv_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

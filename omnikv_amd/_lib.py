@@ -32,6 +32,8 @@ EXPORTS = (
     "okv_noalloc_scratch_bytes",
     "okv_gather_rows",
     "okv_offload_stage",
+    "okv_offload_plan",
+    "okv_offload_fetch",
 )
 
 
@@ -107,6 +109,10 @@ def _declare(l):
     l.okv_noalloc_scratch_bytes.argtypes = []
     l.okv_gather_rows.restype = C.c_int
     l.okv_gather_rows.argtypes = [vp, C.POINTER(KVLayout), vp, i64, vp, i32, i32, vp, i64, i64, i64, vp]
+    l.okv_offload_plan.restype = C.c_int
+    l.okv_offload_plan.argtypes = [vp, i32, vp, vp, i32, vp, vp, vp, vp]
+    l.okv_offload_fetch.restype = C.c_int
+    l.okv_offload_fetch.argtypes = [vp, i64, vp, vp, vp, i32, vp, vp]
     l.okv_offload_stage.restype = C.c_int
     l.okv_offload_stage.argtypes = [vp, i64, vp, i32, vp, i32, vp, vp, vp]
 

@@ -103,8 +103,11 @@ class OmniKVMultiStageCache:
         self.need_cat_layers = []
         self.device = "cpu" if real_offload else None
         self.real_offload = bool(real_offload)
-        if offload_mode not in ("memcpy", "zero_copy"):
-            raise ValueError("offload_mode must be 'memcpy' or 'zero_copy'")
+        if offload_mode not in ("memcpy", "zero_copy", "incremental"):
+            raise ValueError("offload_mode must be 'memcpy', 'zero_copy' or 'incremental'")
+        if offload_mode == "incremental" and not self._stage_at_selection:
+            raise ValueError("incremental staging plans one exchange per selection for the whole group of layers; "
+                             "a cache that stages layer by layer at layer time takes 'zero_copy' or 'memcpy'")
         self.offload_mode = offload_mode
         self.cpu_num_threads = int(cpu_num_threads)
         self.max_new_tokens = int(max_new_tokens)
@@ -126,6 +129,7 @@ class OmniKVMultiStageCache:
         self._part_src: Dict[int, int] = {}        # sparse layer -> selection number it was gathered with
         self._staged_for: Dict[int, int] = {}      # sparse layer -> selection number its rows were staged with
         self._staging: Dict[int, torch.Tensor] = {}
+        self._plan: Dict[int, Dict[str, torch.Tensor]] = {}  # filter layer -> slot maps of its group (incremental mode)
         self._events: Dict[int, torch.cuda.Event] = {}
         self._recorded: Dict[int, threading.Event] = {}
         self._copy_stream: Optional[torch.cuda.Stream] = None
@@ -172,8 +176,8 @@ class OmniKVMultiStageCache:
         preallocated.  With real_offload only the zero-copy mode qualifies: there the GPU
         fetches the selected pinned rows itself, on the copy stream, and the fork and join of
         that stream become part of the graph; the memcpy mode packs rows on host threads."""
-        if self.real_offload and self.offload_mode != "zero_copy":
-            raise NotImplementedError("static decode with real_offload needs offload_mode='zero_copy'")
+        if self.real_offload and self.offload_mode == "memcpy":
+            raise NotImplementedError("static decode with real_offload needs offload_mode='zero_copy' or 'incremental'")
         if self._static:
             return
         any_store = next(iter(self._store.values()))
@@ -390,6 +394,13 @@ class OmniKVMultiStageCache:
             self._recorded[i] = threading.Event()
             if i not in self._events:
                 self._events[i] = torch.cuda.Event()
+        if self.offload_mode == "incremental":
+            self._copy_stream.wait_stream(torch.cuda.current_stream(dev))
+            with torch.cuda.stream(self._copy_stream):
+                self._stage_incremental(idx32, layers)
+                for i in layers:
+                    self._recorded[i].set()
+            return
         if self.offload_mode == "zero_copy":
             # the GPU reads the pinned rows itself: one gather per layer on the copy stream
             self._copy_stream.wait_stream(torch.cuda.current_stream(dev))
@@ -424,6 +435,44 @@ class OmniKVMultiStageCache:
         self._worker = threading.Thread(target=work, daemon=True)
         self._worker.start()
 
+    def _stage_incremental(self, idx32: torch.Tensor, layers: List[int]) -> None:
+        """On the current (copy) stream: plan which rows the new selection does not find staged and
+        which slots the dropped rows free (okv_offload_plan, once for the group), then fetch those
+        rows of every layer from pinned memory into the freed slots (okv_offload_fetch) and record
+        the layer's event.  Nothing here touches the host; the row count lives on the device."""
+        sel = self.layer_state[layers[0]][1]
+        dev, k = idx32.device, idx32.shape[1]
+        n_tok = self._host_kv[layers[0]].shape[0]
+        plan = self._plan.get(sel)
+        if plan is None or plan["slot_tok"].shape[0] != k or plan["slot_of"].shape[0] != n_tok:
+            plan = {"slot_tok": torch.full((k,), -1, dtype=torch.int32, device=dev),
+                    "slot_of": torch.full((n_tok,), -1, dtype=torch.int32, device=dev),
+                    "fetch_tok": torch.empty((k,), dtype=torch.int32, device=dev),
+                    "fetch_slot": torch.empty((k,), dtype=torch.int32, device=dev),
+                    "fetch_count": torch.zeros((1,), dtype=torch.int32, device=dev)}
+            self._plan[sel] = plan
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        check(lib().okv_offload_plan(idx32.data_ptr(), k, plan["slot_tok"].data_ptr(), plan["slot_of"].data_ptr(), n_tok,
+                                     plan["fetch_tok"].data_ptr(), plan["fetch_slot"].data_ptr(),
+                                     plan["fetch_count"].data_ptr(), stream))
+        for i in layers:
+            host = self._host_kv[i]
+            part = self._part.get(i)
+            if part is None or part.shape[1] != k:
+                part = torch.empty((1, k) + tuple(host.shape[1:]), dtype=host.dtype, device=dev)
+                self._part[i] = part
+            if i not in self._events:
+                self._events[i] = torch.cuda.Event()
+            check(lib().okv_offload_fetch(host.data_ptr(), host.stride(0) * host.element_size(), plan["fetch_tok"].data_ptr(),
+                                          plan["fetch_slot"].data_ptr(), plan["fetch_count"].data_ptr(), k,
+                                          part.data_ptr(), stream))
+            self._events[i].record(torch.cuda.current_stream(dev))
+
+    def last_fetch_count(self, sel_layer_idx: int) -> int:
+        """Rows per layer the latest selection of this filter layer had to fetch over the host link
+        (incremental mode); synchronises with the device."""
+        return int(self._plan[sel_layer_idx]["fetch_count"].item())
+
     def _stage_static(self, sel_layer_idx: int, idx32: torch.Tensor) -> None:
         """Static decode with the host tier: the copy stream gathers the selected pinned rows
         of every layer of the group (the GPU reads host memory itself), one event per layer.
@@ -436,6 +485,10 @@ class OmniKVMultiStageCache:
         if self._copy_stream is None:
             self._copy_stream = torch.cuda.Stream(device=dev)
         self._copy_stream.wait_stream(torch.cuda.current_stream(dev))
+        if self.offload_mode == "incremental":
+            with torch.cuda.stream(self._copy_stream):
+                self._stage_incremental(idx32, list(range(lo, hi)))
+            return
         with torch.cuda.stream(self._copy_stream):
             for i in range(lo, hi):
                 host = self._host_kv[i]
@@ -472,6 +525,10 @@ class OmniKVMultiStageCache:
         if self._part_src.get(layer_idx) != self._sel_gen[sel]:
             if self.real_offload:
                 part = self._wait_part(layer_idx)
+                if self.offload_mode == "incremental":
+                    # the staged rows are a set; the reference hands them out in ascending token order
+                    order = self._plan[sel]["slot_of"][idx32[0].long()].long()
+                    part = part.index_select(1, order)
                 pk = part[:, :, 0].permute(0, 2, 1, 3)
                 pv = part[:, :, 1].permute(0, 2, 1, 3)
             else:

@@ -29,7 +29,7 @@ def main():
     ap.add_argument("--selector", default="last")
     ap.add_argument("--select-layers", default="2,8,18")
     ap.add_argument("--real-offload", action="store_true")
-    ap.add_argument("--offload-mode", default="zero_copy", choices=["zero_copy", "memcpy"])
+    ap.add_argument("--offload-mode", default="zero_copy", choices=["zero_copy", "memcpy", "incremental"])
     ap.add_argument("--full-attention", action="store_true", help="no selection: every layer attends to everything")
     ap.add_argument("--graph", action="store_true", help="replay the decode step from a HIP graph")
     ap.add_argument("--trace", default=None, metavar="DESC",

@@ -141,7 +141,7 @@ def test_cache_matches_reference_semantics_on_gpu(dtype):
     assert dut.device is None
 
 
-@pytest.mark.parametrize("mode", ["memcpy", "zero_copy"])
+@pytest.mark.parametrize("mode", ["memcpy", "zero_copy", "incremental"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_cache_with_host_offload_tier(dtype, mode):
     dut = _run_decode(dtype, real_offload=True, offload_mode=mode)
@@ -201,6 +201,73 @@ def test_without_pack_cache_fetches_rows_per_layer(real_offload, mode):
         dut._join_worker()
     else:
         assert staged == []
+
+
+@pytest.mark.parametrize("overlap", [0.0, 0.5, 0.9, 1.0])
+def test_incremental_staging_fetches_only_rows_that_are_new(overlap):
+    """offload_mode='incremental': consecutive selections that share a fraction `overlap` of their
+    tokens.  After every selection the staged rows are exactly the selected set, only the rows
+    the previous selection did not hold crossed the host link, every sparse layer's attention
+    matches the oracle cache (which gathers everything anew, modeling/spec_cache.py:290-306), and
+    update() still hands out the reference's tensors in the reference's order."""
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(int(overlap * 100) + 3)
+    n, kk, L, hq, hkv, d = 5000, 500, 6, 32, 8, 128
+    full = orc.full_attn_layers_from_select_layers([0], L)  # filter 0, wait 1, sparse 2..5
+    ref = orc.OracleMultiStageCache(full, L, 1, True)
+    dut = OmniKVMultiStageCache(full, L, 1, True, max_new_tokens=16, offload_mode="incremental")
+    for i in range(L):
+        k = torch.randn((1, hkv, n, d), generator=g).to(dtype)
+        v = torch.randn((1, hkv, n, d), generator=g).to(dtype)
+        ref.update(k, v, i)
+        dut.update(k.to(DEV), v.to(DEV), i)
+    ref.stage = dut.stage = "decoding"
+    sparse = [i for i, st in dut.layer_state.items() if st[0]]
+    assert sparse == [2, 3, 4, 5]
+    prev = None
+    for step in range(4):
+        if prev is None:
+            idx = torch.randperm(n, generator=g)[:kk].sort().values
+        else:
+            keep = prev[torch.randperm(kk, generator=g)[: int(round(overlap * kk))]]
+            rest = torch.tensor(sorted(set(range(n)) - set(prev.tolist())))
+            fresh = rest[torch.randperm(len(rest), generator=g)[: kk - len(keep)]]
+            idx = torch.cat([keep, fresh]).sort().values
+        ref.set_idx_on_gpu(idx[None], 0)
+        dut.set_idx_on_gpu(idx[None].to(DEV), 0)
+        expect_fetch = kk if prev is None else kk - len(set(idx.tolist()) & set(prev.tolist()))
+        for i in range(L):
+            q = torch.randn((1, hq, 1, d), generator=g).to(dtype)
+            k = torch.randn((1, hkv, 1, d), generator=g).to(dtype)
+            v = torch.randn((1, hkv, 1, d), generator=g).to(dtype)
+            rk, rv = ref.update(k, v, i)
+            want = orc.gqa_attention(q.float(), rk.float(), rv.float())[:, :, 0]
+            dut.append(k.to(DEV), v.to(DEV), i)
+            out = dut.attend(q.to(DEV), i).cpu().float()
+            assert (out - want).abs().max() < TOL[dtype], (step, i)
+        assert dut.last_fetch_count(0) == expect_fetch, step
+        plan = dut._plan[0]
+        assert torch.equal(plan["slot_tok"].cpu().sort().values.long(), idx)  # the staged set is the selection
+        assert torch.equal(plan["slot_of"].cpu()[idx].sort().values, torch.arange(kk, dtype=torch.int32))
+        assert int((plan["slot_of"] >= 0).sum()) == kk
+        for i in sparse:  # the staged rows themselves: slot s holds token slot_tok[s]'s K and V
+            st = plan["slot_tok"].cpu().long()
+            assert torch.equal(dut._part[i][0, :, 0].cpu(), ref.key_cache[i][0, :, st].permute(1, 0, 2))
+            assert torch.equal(dut._part[i][0, :, 1].cpu(), ref.value_cache[i][0, :, st].permute(1, 0, 2))
+        prev = idx
+    # reference-style consumption: update() returns gathered rows ++ tail in ascending token order
+    for i in range(L):
+        k = torch.randn((1, hkv, 1, d), generator=g).to(dtype)
+        v = torch.randn((1, hkv, 1, d), generator=g).to(dtype)
+        rk, rv = ref.update(k, v, i)
+        dk, dv = dut.update(k.to(DEV), v.to(DEV), i)
+        assert torch.equal(dk.cpu(), rk) and torch.equal(dv.cpu(), rv), i
+
+
+def test_incremental_staging_is_refused_where_layers_stage_themselves():
+    from omnikv_amd.cache import WOPackCache
+    with pytest.raises(ValueError, match="incremental"):
+        WOPackCache([0, 4], 4, 1, True, offload_mode="incremental")
 
 
 def test_lazy_reselection_skips_similar_selections():

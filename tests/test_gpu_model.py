@@ -140,23 +140,25 @@ def test_generate_greedy_and_error_paths():
         lm2.forward(ids[:, :1], cache)
 
 
-@pytest.mark.parametrize("selector_cls,offload", [("last", False), ("softmax_before_last", False), ("last", True)])
+@pytest.mark.parametrize("selector_cls,offload", [("last", False), ("softmax_before_last", False), ("last", True),
+                                                  ("last", "incremental")])
 def test_graph_replayed_decode_matches_eager(selector_cls, offload):
     """A decode step captured in a HIP graph (device-side lengths and positions; with the
     host tier also the copy stream's zero-copy gathers) must reproduce the eager path
     token for token and logit for logit on every replay."""
     ids = torch.randint(0, SHAPE.vocab_size, (1, 400), generator=torch.Generator().manual_seed(4)).to(DEV)
     steps = 7
+    kw = {"offload_mode": offload} if isinstance(offload, str) else {}  # a string names the staging mode of the tier
 
     def fresh():
-        lm = OmniKVMulLM(SHAPE, _config(selector_cls, offload)).float().to(DEV)
+        lm = OmniKVMulLM(SHAPE, _config(selector_cls, bool(offload))).float().to(DEV)
         lm.init_weights(seed=11, std=0.08)
         return lm
 
     lm = fresh()
-    eager_toks, eager_logits = lm.generate_greedy(ids, steps + 4, max_new_tokens=32)
+    eager_toks, eager_logits = lm.generate_greedy(ids, steps + 4, max_new_tokens=32, **kw)
     lm2 = fresh()
-    logits, cache = lm2.forward(ids, None, max_new_tokens=32)
+    logits, cache = lm2.forward(ids, None, max_new_tokens=32, **kw)
     assert torch.equal(logits, eager_logits[0])
     tok = logits[:, -1].argmax(-1, keepdim=True)
     graph, token, glogits = lm2.capture_decode(cache, tok, warmup=2)  # two eager static steps, then capture
