@@ -90,10 +90,13 @@ def main():
     if args.real_offload:
         cache._join_worker()
     extra = {}
+    if args.real_offload and args.offload_mode == "incremental" and not args.full_attention:
+        # rows per layer the last selection of each filter layer had to fetch (of `selected`)
+        extra["rows_fetched_per_layer_last_step"] = {str(f): cache.last_fetch_count(f) for f in sorted(cache._plan)}
     if tracer is not None:
         mass, _ = tracer.matrices()
         layers, quality = trace.suggest_filter_layers(mass, num_filters=len(args.select_layers.split(",")))
-        extra = {"trace_file": tracer.save_idx(), "suggested_select_layers": layers, "suggested_quality": quality,
+        extra = {**extra, "trace_file": tracer.save_idx(), "suggested_select_layers": layers, "suggested_quality": quality,
                  "configured_quality": trace.schedule_quality(mass, [int(i) for i in args.select_layers.split(",")])[0]}
     print(json.dumps({
         **extra,

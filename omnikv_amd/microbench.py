@@ -25,7 +25,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--op", required=True,
                     choices=["dense", "fused", "score", "topk", "sparse", "sparse_packed", "sparse_floor", "empty", "gather", "copy",
-                             "offload_memcpy", "offload_zero_copy", "h2d", "window", "window_loop",
+                             "offload_memcpy", "offload_zero_copy", "offload_incremental", "h2d", "window", "window_loop",
                              "paged_dense", "paged_fused", "paged_score", "paged_topk", "paged_sparse", "paged_sparse_slots"])
     ap.add_argument("--batch", type=int, default=16, help="requests of the paged_* ops (ragged lengths 8192..32768)")
     ap.add_argument("--page-size", type=int, default=16)
@@ -34,6 +34,8 @@ def main():
                     help="paged_* ops: the same ragged batch in (bsz, Hkv, Nmax, D) tensors, no page table")
     ap.add_argument("--window", type=int, default=16, help="query positions of the window selectors")
     ap.add_argument("--cpu-threads", type=int, default=8, help="packing threads of the offload tier")
+    ap.add_argument("--overlap", type=float, default=0.9,
+                    help="offload_incremental: share of a selection's tokens that the previous selection already held")
     ap.add_argument("--ctx", type=int, default=131072)
     ap.add_argument("--ratio", type=float, default=0.067)
     ap.add_argument("--tail", type=int, default=1)
@@ -90,7 +92,8 @@ def main():
         # one offloaded layer group: `nl` layers whose prompt K/V live in pinned host memory
         from .cache import OmniKVMultiStageCache
         off = OmniKVMultiStageCache([0, nl + 2], nl + 2, num_wait_load_layers=1, real_offload=True,
-                                    offload_mode="zero_copy" if args.op == "offload_zero_copy" else "memcpy",
+                                    offload_mode={"offload_zero_copy": "zero_copy", "offload_incremental": "incremental"}.get(
+                                        args.op, "memcpy"),
                                     cpu_num_threads=args.cpu_threads)
         for l in range(nl + 2):
             off.append(ks[l % nl][:, :, :n], vs[l % nl][:, :, :n], l)
@@ -99,6 +102,21 @@ def main():
         if args.op == "h2d":
             hsrc = torch.empty(k_sel * 2 * HKV * D * es, dtype=torch.uint8).pin_memory()
             hdst = torch.empty(k_sel * 2 * HKV * D * es, dtype=torch.uint8, device=dev)
+        if args.op == "offload_incremental":
+            # a chain of selections, each keeping `overlap` of the previous one's tokens (seeded, on the device)
+            gsel = torch.Generator(device=dev).manual_seed(5)
+            keep_n = int(round(args.overlap * k_sel))
+            sels = [idx]
+            for _ in range(args.warmup + args.reps + 1):
+                prev = sels[-1][0].long()
+                held = torch.zeros(n, dtype=torch.bool, device=dev)
+                held[prev] = True
+                keep = prev[torch.randperm(k_sel, generator=gsel, device=dev)[:keep_n]]
+                rest = torch.nonzero(~held)[:, 0]
+                fresh = rest[torch.randperm(rest.numel(), generator=gsel, device=dev)[: k_sel - keep_n]]
+                sels.append(torch.cat([keep, fresh]).sort().values.to(torch.int32)[None].contiguous())
+            off.set_idx_on_gpu(sels[0], 0)  # the first selection fetches everything; not timed
+            torch.cuda.synchronize()
 
     floor = None
     if args.op in ("sparse_floor", "empty"):
@@ -152,7 +170,7 @@ def main():
             return hdst.copy_(hsrc, non_blocking=True)
         if off is not None:
             # select once, stage the rows of all `nl` layers, wait for the last of them
-            off.set_idx_on_gpu(idx, 0)
+            off.set_idx_on_gpu(sels[i + 1] if args.op == "offload_incremental" else idx, 0)
             for l2 in range(2, nl + 2):
                 off._wait_part(l2)
             return None
@@ -174,6 +192,7 @@ def main():
         "h2d": 2.0 * k_sel * row,
         "offload_memcpy": 2.0 * k_sel * row * nl,
         "offload_zero_copy": 2.0 * k_sel * row * nl,
+        "offload_incremental": 2.0 * (k_sel - int(round(args.overlap * k_sel))) * row * nl,  # rows that are new
     }[args.op]
     stream = torch.cuda.current_stream()
     for i in range(args.warmup):
@@ -182,13 +201,19 @@ def main():
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record(stream)
     for i in range(args.reps):
-        call(i)
+        call(args.warmup + i)
     e1.record(stream)
     e1.synchronize()
     us = e0.elapsed_time(e1) * 1e3 / args.reps
-    print(json.dumps({"op": args.op, "ctx": n, "selected": k_sel, "tail": tail, "dtype": args.dtype,
-                      "layout": args.layout, "us_per_call": us, "algorithmic_bytes": algo,
-                      "algorithmic_GBps": algo / us / 1e3, "frac_of_8TBps": algo / us / 1e3 / 8000.0}))
+    res = {"op": args.op, "ctx": n, "selected": k_sel, "tail": tail, "dtype": args.dtype,
+           "layout": args.layout, "us_per_call": us, "algorithmic_bytes": algo,
+           "algorithmic_GBps": algo / us / 1e3 if algo else None, "frac_of_8TBps": algo / us / 1e3 / 8000.0}
+    if args.op.startswith("offload"):
+        res.update({"layers_per_selection": nl, "host_link_GBps": algo / us / 1e3})
+        if args.op == "offload_incremental":
+            res.update({"overlap": args.overlap, "rows_fetched_per_layer": off.last_fetch_count(0),
+                        "full_restage_bytes": 2.0 * k_sel * row * nl})
+    print(json.dumps(res))
 
 
 def paged(args, dev):
