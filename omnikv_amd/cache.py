@@ -576,6 +576,38 @@ class OmniKVMultiStageCache:
         kview, vview = self._store[layer_idx].views()
         return ops.dense_attn(query_states, kview, vview, scale=scale)
 
+    def select_with_query(self, query_states: torch.Tensor, layer_idx: int, num_selected_tokens: int,
+                          consider_len: int, selector_cls: str, forced_tail: int = 0) -> torch.Tensor:
+        """Filter layer with a selector that scores separately from the layer's attention (the
+        window selectors `uniform` / `exp`, modeling/omnikv.py:59-105,177-210): scores of the first
+        `consider_len` cached tokens from the rotated query block (bsz, Hq, W, D), top-k, the last
+        `forced_tail` prompt positions appended (the window still inside the prompt), then
+        set_idx_on_gpu.  In static decode everything has a fixed shape and lands in a fixed index
+        buffer, so the step can be captured.  Returns the int32 (bsz, k) selection."""
+        from . import selector
+        if not self._static:
+            idx = selector.select_from_query(query_states, self.key_cache[layer_idx], num_selected_tokens, consider_len,
+                                             selector_cls)
+            if forced_tail:
+                end = consider_len + forced_tail
+                tail_idx = torch.arange(end - forced_tail, end, device=idx.device)
+                idx = torch.cat([idx, tail_idx[None, :].repeat(idx.shape[0], 1)], dim=1)
+            self.set_idx_on_gpu(idx, layer_idx)
+            return self._idx[layer_idx]
+        if forced_tail:
+            raise RuntimeError("static decode with a window selector starts once the window has left the prompt")
+        scores = selector.score_from_query(query_states, self._store[layer_idx].k, consider_len, selector_cls)
+        k = min(num_selected_tokens, consider_len)
+        buf = self._idx.get(layer_idx)
+        if buf is None or buf.shape[1] != k:
+            buf = torch.empty((scores.shape[0], k), dtype=torch.int32, device=scores.device)
+            self._idx[layer_idx] = buf  # the sparse layers keep reading this very buffer
+        ops.topk(scores, k, out=buf)
+        self._sel_gen[layer_idx] = self._sel_gen.get(layer_idx, 0) + 1
+        if self.real_offload:
+            self._stage_static(layer_idx, buf)
+        return buf
+
     def attend_and_select(self, query_states: torch.Tensor, layer_idx: int, num_selected_tokens: int,
                           consider_len: int, selector_cls: str = "last", scale: Optional[float] = None):
         """Filter layer: dense attention and the filter-layer scores in one pass over

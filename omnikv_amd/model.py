@@ -153,19 +153,20 @@ class OmniKVMulLayer(nn.Module):
                                                             self.selector_cls)
                 else:
                     forced = max(0, self.window_size - self.decode_step)
-                    self.hidden_state_window = torch.cat([self.hidden_state_window, hidden_states], dim=1)[
-                        :, -self.window_size:]
+                    if getattr(past_key_value, "_static", False):
+                        # in place (one fixed buffer per layer), so that a captured step finds on replay
+                        # what the previous replay left
+                        self.hidden_state_window.copy_(torch.cat([self.hidden_state_window[:, 1:], hidden_states], dim=1))
+                    else:
+                        self.hidden_state_window = torch.cat([self.hidden_state_window, hidden_states], dim=1)[
+                            :, -self.window_size:].contiguous()
                     win = self.hidden_state_window
                     # every window row is rotated with the CURRENT position (modeling/omnikv.py:34-35)
                     wq = attn.q_proj(win).view(win.shape[0], win.shape[1], attn.num_heads, attn.head_dim).transpose(1, 2)
                     cos, sin = attn.rotary_emb(wq, position_ids)
                     wq, _ = apply_rotary_pos_emb(wq, wq, cos, sin)
-                    kview = past_key_value.key_cache[self.layer_idx]
-                    idx = select_from_query(wq.contiguous(), kview, max(1, num_selected_tokens - forced),
-                                            consider_len - forced, self.selector_cls)
-                    tail_idx = torch.arange(self.prefill_len - forced, self.prefill_len, device=idx.device)
-                    idx = torch.cat([idx, tail_idx[None, :].repeat(idx.shape[0], 1)], dim=1)
-                    past_key_value.set_idx_on_gpu(idx, self.layer_idx)
+                    past_key_value.select_with_query(wq.contiguous(), self.layer_idx, max(1, num_selected_tokens - forced),
+                                                     consider_len - forced, self.selector_cls, forced_tail=forced)
                     o = past_key_value.attend(q, self.layer_idx)
                 past_key_value.stage = "decoding"
                 self.decode_step += 1
@@ -263,13 +264,22 @@ class OmniKVMulLM(nn.Module):
         """Capture one greedy decode step in a HIP graph.  Returns (graph, token, logits):
         each graph.replay() consumes `token` (1, 1), writes the step's fp32 logits into
         `logits` and the argmax back into `token`, and moves every length on the device
-        by one -- a generation loop with no host work per token besides the replay."""
-        if "last" not in self.config.get("selector_cls", "softmax_before_last"):
-            raise NotImplementedError("the window selectors keep a host-side window; capture the `last` family")
+        by one -- a generation loop with no host work per token besides the replay.
+        Before the capture `warmup` eager steps run (after, for the window selectors, as many
+        as the query window needs to leave the prompt): `token` is the one they ended on."""
         if trace.idx_tracer is not None:
             raise RuntimeError("selection tracing keeps per-step host state; trace an eager run")
-        cache.enable_static_decode()
         token = first_token.clone().view(1, 1)
+        if "last" not in self.config.get("selector_cls", "softmax_before_last"):
+            # the window selectors force-keep the last prompt positions until the query window has left
+            # the prompt (modeling/omnikv.py:177-210): those steps change shape and run eagerly first
+            sel_layers = [l for l in self.model.layers if l.layer_idx in l.do_select_layers]
+            if any(l.hidden_state_window is None or l.hidden_state_window.shape[1] < l.window_size for l in sel_layers):
+                raise NotImplementedError("a captured step needs a full query window: the prompt is shorter than window_size")
+            for _ in range(max([0] + [l.window_size - l.decode_step for l in sel_layers])):
+                logits, _ = self.forward(token, cache)
+                token.copy_(logits[:, -1].argmax(-1, keepdim=True))
+        cache.enable_static_decode()
         stream = torch.cuda.Stream(device=token.device)
         stream.wait_stream(torch.cuda.current_stream(token.device))
         with torch.cuda.stream(stream):
