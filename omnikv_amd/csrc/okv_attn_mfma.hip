@@ -313,6 +313,19 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
         load_tile(tr, kB, vB);
         compute(t, kA, vA);
         compute(t + 64, kB, vB);
+      } else if (!KLDS && t + 128 == t_last) {
+        // three tiles (a sparse layer's usual share): a third set of registers keeps all of them in
+        // flight behind one index round trip, instead of the third tile waiting for the first
+        uint4 kC[4], vC[4];
+        TileRows tr2;
+        tile_rows(t + 64, tr);
+        tile_rows(t + 128, tr2);
+        load_tile(tr0, kA, vA);
+        load_tile(tr, kB, vB);
+        load_tile(tr2, kC, vC);
+        compute(t, kA, vA);
+        compute(t + 64, kB, vB);
+        compute(t + 128, kC, vC);
       } else {
         tile_rows(t + 64, tr);  // both lookups leave before the first one is awaited
         load_tile(tr0, kA, vA);

@@ -91,9 +91,11 @@ class _OracleRunner:
 
 
 @pytest.mark.parametrize("selector_cls", ["last", "softmax_before_last", "uniform", "exp"])
-@pytest.mark.parametrize("real_offload", [False, True])
+@pytest.mark.parametrize("real_offload", [False, True, "incremental", "memcpy"])
 def test_greedy_decode_matches_oracle(selector_cls, real_offload):
     torch.manual_seed(0)
+    mode = {"offload_mode": real_offload} if isinstance(real_offload, str) else {}  # a string names the tier's staging mode
+    real_offload = bool(real_offload)
     cfg = _config(selector_cls, real_offload)
     lm = OmniKVMulLM(SHAPE, cfg).float()
     lm.init_weights(seed=3, std=0.08)
@@ -102,7 +104,7 @@ def test_greedy_decode_matches_oracle(selector_cls, real_offload):
     n, steps = 500, 6
     ids = torch.randint(0, SHAPE.vocab_size, (1, n), generator=torch.Generator().manual_seed(1))
     want = ref.forward(ids)
-    got, cache = dut.forward(ids.to(DEV), None, max_new_tokens=16, cpu_num_threads=2)
+    got, cache = dut.forward(ids.to(DEV), None, max_new_tokens=16, cpu_num_threads=2, **mode)
     assert got.shape == (1, 1, SHAPE.vocab_size) and got.dtype == torch.float32
     assert (got.cpu() - want).abs().max() < 2e-3
     dense = sorted(i for i, s in cache.layer_state.items() if not s[0])
