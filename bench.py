@@ -87,80 +87,50 @@ def build_cache(n, tail_cap, dtype, device, layout):
     return ks, vs, qs
 
 
-def make_step(ks, vs, qs, n, tail, k_sel, selector):
+def make_step(ks, vs, qs, n, tail, k_sel, selector, overlap_select=False):
+    """One decode step's attention over the 32 layers.  With overlap_select the top-k of a filter layer runs
+    on a stream of its own under the wait-load layer that follows it -- only the group's sparse layers need its
+    result, which is what num_wait_load_layers is for (modeling/spec_cache.py:271-281) -- and the first sparse
+    layer of the group waits for it.  Measured, the replayed graph is SLOWER that way (1.197 against 1.166 ms per
+    step at 128K: three forks and joins cost more than the 3 x 18 us they hide, and the top-k's workgroups slow
+    the dense pass they run beside), so it is off unless asked for.  Scores and indices live in fixed buffers."""
     from omnikv_amd import ops
 
     kinds = schedule()
+    dev = ks[0].device
+    side = torch.cuda.Stream(device=dev) if overlap_select else None
+    scores = {l: torch.empty((1, n), dtype=torch.float32, device=dev) for l in FILTER_LAYERS}
+    idx = {l: torch.empty((1, min(k_sel, n)), dtype=torch.int32, device=dev) for l in FILTER_LAYERS}
+    done = {l: torch.cuda.Event() for l in FILTER_LAYERS}
 
     def step():
-        idx = {}
         outs = []
+        main = torch.cuda.current_stream(dev)
+        waited = set()
         for l in range(LAYERS):
             kind, src = kinds[l]
             kfull, vfull = ks[l][:, :, : n + tail], vs[l][:, :, : n + tail]
             if kind == "dense":
                 outs.append(ops.dense_attn(qs[l], kfull, vfull))
             elif kind == "filter":
-                o, sc = ops.dense_attn(qs[l], kfull, vfull, selector=selector, score_len=n)
-                idx[l] = ops.topk(sc, k_sel)
+                o, sc = ops.dense_attn(qs[l], kfull, vfull, selector=selector, score_len=n, scores_out=scores[l])
                 outs.append(o)
+                if side is None:
+                    ops.topk(sc, k_sel, out=idx[l])
+                else:
+                    side.wait_stream(main)
+                    with torch.cuda.stream(side):
+                        ops.topk(sc, k_sel, out=idx[l])
+                        done[l].record(side)
             else:
+                if side is not None and src not in waited:
+                    main.wait_event(done[src])
+                    waited.add(src)
                 outs.append(ops.sparse_attn(qs[l], ks[l][:, :, :n], vs[l][:, :, :n], idx=idx[src],
                                             tail_k=ks[l][:, :, n: n + tail], tail_v=vs[l][:, :, n: n + tail]))
         return outs, idx
 
     return step
-
-
-def cpu_baseline(n, k_sel, selector, budget_s=25.0):
-    """The CPU oracle on this host: one dense layer, one filter layer (score +
-    top-k + dense attention) and one sparse layer (gather + cat + attention) at
-    the benchmark's context length in fp32, scaled to the 32-layer schedule."""
-    from omnikv_amd import synth
-    from oracle import okv_oracle as orc
-
-    cores = os.cpu_count() or 1
-    torch.set_num_threads(cores)
-    q, k, v = synth.filter_layer_inputs(n, HQ, HKV, D)
-    qn = synth.fresh_q()
-    tk, tv = torch.randn(1, HKV, 1, D), torch.randn(1, HKV, 1, D)
-
-    def t(fn, reps):
-        best = []
-        for _ in range(reps):
-            s = time.perf_counter()
-            r = fn()
-            best.append(time.perf_counter() - s)
-        best.sort()
-        return best[len(best) // 2], r
-
-    t0 = time.perf_counter()
-    dense_s, _ = t(lambda: orc.gqa_attention(q, k, v), 1)
-    reps = 3 if (time.perf_counter() - t0) * 8 < budget_s else 1
-    dense_s, _ = t(lambda: orc.gqa_attention(q, k, v), reps)
-    score_s, sc = t(lambda: orc.score_tokens(q, k, n, selector), reps)
-    topk_s, idx = t(lambda: orc.select_topk(sc, k_sel), reps)
-
-    def sparse():
-        pk = torch.cat([orc.gather_rows(k, idx[0]), tk], dim=-2)
-        pv = torch.cat([orc.gather_rows(v, idx[0]), tv], dim=-2)
-        return orc.gqa_attention(qn, pk, pv)
-
-    sparse_s, _ = t(sparse, max(reps, 3))
-    kinds = schedule()
-    nd = sum(1 for x in kinds.values() if x[0] in ("dense", "filter"))
-    nf = sum(1 for x in kinds.values() if x[0] == "filter")
-    ns = sum(1 for x in kinds.values() if x[0] == "sparse")
-    step_s = nd * dense_s + nf * (score_s + topk_s) + ns * sparse_s
-    return {
-        "value": step_s * 1e6 / LAYERS,
-        "unit": "us/layer",
-        "cores": cores,
-        "kind": "port",
-        "sample": (f"torch fp32 CPU oracle at N={n}: 1 dense layer {dense_s*1e3:.1f} ms, score {score_s*1e3:.1f} ms, "
-                   f"top-k {topk_s*1e3:.2f} ms, 1 sparse layer (gather+cat+attention, k={k_sel}) {sparse_s*1e3:.2f} ms; "
-                   f"median of {reps}; scaled to {nd} dense + {nf} score/top-k + {ns} sparse layers"),
-    }
 
 
 def time_graph(fn, launches, reps, stream):
@@ -339,6 +309,8 @@ def main():
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32"])
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--overlap-select", action="store_true",
+                    help="run each filter layer's top-k on a stream of its own under the wait-load layer (measured slower)")
     ap.add_argument("--no-variants", action="store_true", help="skip the extra steps (selector last, k = round(ratio N))")
     ap.add_argument("--split-rows", type=int, default=0, help="override rows per split (0 = automatic)")
     ap.add_argument("--attn-variant", type=int, default=0, help="1 = portable VALU stage 1 for every dtype")
@@ -361,7 +333,7 @@ def main():
     n, tail = args.ctx, args.tail
     k_sel = int(args.ratio * n)  # the reference truncates: modeling/omnikv.py:169-171
     ks, vs, qs = build_cache(n, max(tail, 1), dtype, device, args.layout)
-    step = make_step(ks, vs, qs, n, tail, k_sel, args.selector)
+    step = make_step(ks, vs, qs, n, tail, k_sel, args.selector, args.overlap_select)
 
     stream = torch.cuda.Stream()
     graph = None
@@ -420,7 +392,7 @@ def main():
         if not args.no_variants:
             for name, sel_v, k_v in (("selector_last", "last", k_sel), ("selected_%d" % round(args.ratio * n), args.selector,
                                                                          int(round(args.ratio * n)))):
-                step_v = make_step(ks, vs, qs, n, tail, k_v, sel_v)
+                step_v = make_step(ks, vs, qs, n, tail, k_v, sel_v, args.overlap_select)
                 step_v()
                 stream.synchronize()
                 gv = torch.cuda.CUDAGraph()
@@ -462,6 +434,7 @@ def main():
             "filter_layers": list(FILTER_LAYERS), "num_wait_load_layers": WAIT, "layers": LAYERS,
             "q_heads": HQ, "kv_heads": HKV, "head_dim": D, "kv_layout": args.layout,
             "launch": "hip_graph_replay" if graph is not None else "eager",
+            "topk_stream": "own stream, under the wait-load layer" if args.overlap_select else "main",
             "kv_resident_gb": round(2 * LAYERS * (n + max(tail, 1)) * HKV * D * esize / 1e9, 2),
         },
         "decode_tokens_per_s_attention_only": 1e3 / wall_ms,

@@ -228,7 +228,8 @@ def topk(scores: torch.Tensor, k: int, seq_lens: Optional[torch.Tensor] = None,
 
 def dense_attn(q, k, v=None, seq_len: Optional[int] = None, seq_lens: Optional[torch.Tensor] = None,
                scale: Optional[float] = None, selector: Optional[str] = None,
-               score_len: Optional[int] = None, score_lens: Optional[torch.Tensor] = None):
+               score_len: Optional[int] = None, score_lens: Optional[torch.Tensor] = None,
+               scores_out: Optional[torch.Tensor] = None):
     """Dense GQA decode attention; with `selector` also returns the filter-layer
     scores of the first score_len tokens from the same pass.  okv_dense_attn."""
     q = _q3(q)
@@ -248,7 +249,11 @@ def dense_attn(q, k, v=None, seq_len: Optional[int] = None, seq_lens: Optional[t
         red, norm = _REDUCE[red_s], _NORM[norm_s]
         if score_len is None:
             score_len = seq_len
-        scores = torch.empty((batch, score_len), dtype=torch.float32, device=q.device)
+        scores = scores_out
+        if scores is None:
+            scores = torch.empty((batch, score_len), dtype=torch.float32, device=q.device)
+        elif scores.shape != (batch, score_len) or scores.dtype != torch.float32 or scores.stride(1) != 1:
+            raise ValueError("scores_out must be (bsz, score_len) float32 with contiguous rows")
         sp, ss = scores.data_ptr(), scores.stride(0)
     nbytes = workspace_bytes(_lib.OKV_OP_DENSE_ATTN, batch, hq, lay.num_kv_heads, d, seq_len,
                              with_scores=selector is not None)
