@@ -254,7 +254,7 @@ def measure_kernels(ops, l, check, stream, ks, vs, qs, n, tail, k_sel, selector,
         def floor():
             for layer in sparse_layers:
                 check(l.okv_diag_gather_floor(ks[layer].data_ptr(), vs[layer].data_ptr(), C.byref(lay), any_idx.data_ptr(),
-                                              k_sel, rows_.value, sink.data_ptr(), stream.cuda_stream))
+                                              k_sel, rows_.value, 4, sink.data_ptr(), stream.cuda_stream))
 
         entry("sparse_load_only_floor", "okv::gather_floor_kernel (same grid, index lookups and loads; no arithmetic, no output)",
               time_graph(floor, len(sparse_layers), reps, stream), 2.0 * k_sel * kv_row + 4.0 * k_sel,

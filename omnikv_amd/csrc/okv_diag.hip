@@ -10,7 +10,7 @@ namespace okv {
 // assignment, the index lookup and the two load shapes of attn_stage1_mfma's gather mode (K:
 // lane = row, 4 x 16 bytes of each 64-byte k-step; V: whole 256-byte rows per 16 lanes), every
 // load of up to four tiles in flight at once, and no arithmetic beyond an XOR of what arrived.
-template <int ESIZE>
+template <int TILES>
 __global__ __launch_bounds__(256) void gather_floor_kernel(const char* __restrict__ kb, const char* __restrict__ vb,
                                                            const int32_t* __restrict__ idx, int sel_len,
                                                            int split_rows, int64_t token_bytes, int64_t head_bytes,
@@ -24,7 +24,6 @@ __global__ __launch_bounds__(256) void gather_floor_kernel(const char* __restric
   const char* kh = kb + (int64_t)g * head_bytes;
   const char* vh = vb + (int64_t)g * head_bytes;
   uint32_t acc = 0;
-  constexpr int TILES = 4;
   for (int t0 = begin + wave * 16; t0 < end; t0 += 64 * TILES) {
     int tk[TILES], tv[TILES][4];
 #pragma unroll
@@ -89,20 +88,23 @@ int okv_diag_split_geometry(int op, const okv_shape_t* s, int32_t* split_rows, i
 
 // The load-only counterpart of one okv_sparse_attn launch over rows idx[0 .. sel_len) of a
 // contiguous batch-1 K / V (no tail): same grid (kv heads x splits of split_rows rows), same
-// bytes.  sink: 4 bytes of device memory.
+// bytes; a wave keeps the loads of tiles_in_flight (1, 2 or 4) of its tiles outstanding.  sink: 4 bytes
+// of device memory.
 int okv_diag_gather_floor(const void* k_base, const void* v_base, const okv_kv_layout_t* layout,
-                          const int32_t* idx, int32_t sel_len, int32_t split_rows, void* sink,
-                          okv_stream_t stream) {
+                          const int32_t* idx, int32_t sel_len, int32_t split_rows, int32_t tiles_in_flight,
+                          void* sink, okv_stream_t stream) {
   int rc = validate_layout(layout, k_base, v_base);
   if (rc) return rc;
   OKV_REQUIRE(idx && sink && sel_len >= 1, OKV_ERR_INVALID, "idx, sink or sel_len");
   OKV_REQUIRE(split_rows >= 16 && split_rows % 16 == 0, OKV_ERR_INVALID, "split_rows must be a multiple of 16");
   OKV_REQUIRE(layout->page_table == nullptr && layout->dtype != OKV_F32, OKV_ERR_UNSUPPORTED,
               "the floor kernel reads contiguous 16-bit K/V");
+  OKV_REQUIRE(tiles_in_flight == 1 || tiles_in_flight == 2 || tiles_in_flight == 4, OKV_ERR_INVALID,
+              "tiles_in_flight must be 1, 2 or 4");
   dim3 grid(layout->num_kv_heads, (sel_len + split_rows - 1) / split_rows);
-  hipLaunchKernelGGL(gather_floor_kernel<2>, grid, dim3(256), 0, (hipStream_t)stream, (const char*)k_base,
-                     (const char*)v_base, idx, sel_len, split_rows, layout->token_stride * 2, layout->head_stride * 2,
-                     (uint32_t*)sink);
+  auto kern = tiles_in_flight == 1 ? gather_floor_kernel<1> : tiles_in_flight == 2 ? gather_floor_kernel<2> : gather_floor_kernel<4>;
+  hipLaunchKernelGGL(kern, grid, dim3(256), 0, (hipStream_t)stream, (const char*)k_base, (const char*)v_base, idx,
+                     sel_len, split_rows, layout->token_stride * 2, layout->head_stride * 2, (uint32_t*)sink);
   OKV_HIP_CHECK(hipGetLastError());
   return OKV_OK;
 }

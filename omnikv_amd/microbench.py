@@ -34,6 +34,8 @@ def main():
                     help="paged_* ops: the same ragged batch in (bsz, Hkv, Nmax, D) tensors, no page table")
     ap.add_argument("--window", type=int, default=16, help="query positions of the window selectors")
     ap.add_argument("--cpu-threads", type=int, default=8, help="packing threads of the offload tier")
+    ap.add_argument("--tiles-in-flight", type=int, default=4, choices=[1, 2, 4],
+                    help="sparse_floor: tiles whose loads a wave keeps outstanding")
     ap.add_argument("--overlap", type=float, default=0.9,
                     help="offload_incremental: share of a selection's tokens that the previous selection already held")
     ap.add_argument("--ctx", type=int, default=131072)
@@ -137,7 +139,8 @@ def main():
         if args.op == "sparse_floor":
             rows, sink, lay, C = floor
             return check(lib().okv_diag_gather_floor(ks[l].data_ptr(), vs[l].data_ptr(), C.byref(lay), idx.data_ptr(), k_sel,
-                                                     rows, sink.data_ptr(), torch.cuda.current_stream().cuda_stream))
+                                                     rows, args.tiles_in_flight, sink.data_ptr(),
+                                                     torch.cuda.current_stream().cuda_stream))
         if args.op == "empty":
             return check(lib().okv_diag_empty_launch(floor[1].data_ptr(), torch.cuda.current_stream().cuda_stream))
         if args.op == "dense":
