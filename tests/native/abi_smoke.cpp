@@ -7,6 +7,9 @@
 //   selection      okv_topk on those scores  -> must equal a stable sort of the SAME device scores
 //   sparse layer   okv_sparse_attn over the selected rows + one tail row
 //   bookkeeping    okv_workspace_bytes, okv_gather_rows, error reporting for a bad argument
+//   no allocation  okv_sparse_attn_noalloc must reproduce okv_sparse_attn bit for bit
+//   host tier      okv_offload_plan + okv_offload_fetch over two overlapping selections: the staged
+//                  rows are exactly the second selection, and only its new rows were copied
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
@@ -223,6 +226,79 @@ int main() {
         std::fprintf(stderr, "gathered row %d of head %d differs from its source\n", j, g);
         return 10;
       }
+
+  // ---- the same sparse layer without a workspace: the library's fixed scratch, same bits
+  {
+    void* dout2;
+    HIP_OK(hipMalloc(&dout2, (size_t)HQ * D * 2));
+    OKV(okv_sparse_attn_noalloc(dq, dk, dv, &lay, didx, K_SEL, nullptr, K_SEL, tk, tv, D, (int64_t)rows * D,
+                                (int64_t)HKV * rows * D, nullptr, T, 1, scale, dout2, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    std::vector<uint16_t> out2(HQ * D);
+    HIP_OK(hipMemcpy(out2.data(), dout2, out2.size() * 2, hipMemcpyDeviceToHost));
+    if (out2 != out) {
+      std::fprintf(stderr, "okv_sparse_attn_noalloc differs from okv_sparse_attn\n");
+      return 11;
+    }
+    HIP_OK(hipFree(dout2));
+  }
+
+  // ---- incremental staging: rows of (N, 2, Hkv, D) = one 4 KB row per token (here in device memory; the
+  // tier keeps them in pinned host memory), two selections that share every other token
+  {
+    const int KS = 64;
+    const int64_t row_bytes = 2 * HKV * D * 2;
+    std::vector<uint16_t> hsrc((size_t)N * row_bytes / 2);
+    for (size_t i = 0; i < hsrc.size(); ++i) hsrc[i] = (uint16_t)(i * 2654435761u >> 16);
+    std::vector<int32_t> sel_a(KS), sel_b(KS), minus(KS, -1), minus_n(N, -1);
+    for (int j = 0; j < KS; ++j) sel_a[j] = 7 + 31 * j;                       // ascending, distinct
+    for (int j = 0; j < KS; ++j) sel_b[j] = (j % 2) ? sel_a[j] : sel_a[j] + 5;  // odd entries kept, even ones new
+    void *dsrc, *dstaged;
+    int32_t *dsel, *dslot_tok, *dslot_of, *dftok, *dfslot, *dfcount;
+    HIP_OK(hipMalloc(&dsrc, hsrc.size() * 2));
+    HIP_OK(hipMalloc(&dstaged, (size_t)KS * row_bytes));
+    HIP_OK(hipMalloc((void**)&dsel, KS * 4));
+    HIP_OK(hipMalloc((void**)&dslot_tok, KS * 4));
+    HIP_OK(hipMalloc((void**)&dslot_of, N * 4));
+    HIP_OK(hipMalloc((void**)&dftok, KS * 4));
+    HIP_OK(hipMalloc((void**)&dfslot, KS * 4));
+    HIP_OK(hipMalloc((void**)&dfcount, 4));
+    HIP_OK(hipMemcpy(dsrc, hsrc.data(), hsrc.size() * 2, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dslot_tok, minus.data(), KS * 4, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dslot_of, minus_n.data(), N * 4, hipMemcpyHostToDevice));
+    int32_t fetched[2] = {0, 0};
+    for (int round = 0; round < 2; ++round) {
+      HIP_OK(hipMemcpy(dsel, (round ? sel_b : sel_a).data(), KS * 4, hipMemcpyHostToDevice));
+      OKV(okv_offload_plan(dsel, KS, dslot_tok, dslot_of, N, dftok, dfslot, dfcount, stream));
+      OKV(okv_offload_fetch(dsrc, row_bytes, dftok, dfslot, dfcount, KS, dstaged, stream));
+      HIP_OK(hipStreamSynchronize(stream));
+      HIP_OK(hipMemcpy(&fetched[round], dfcount, 4, hipMemcpyDeviceToHost));
+    }
+    if (fetched[0] != KS || fetched[1] != KS / 2) {
+      std::fprintf(stderr, "incremental staging fetched %d then %d rows, expected %d then %d\n", fetched[0], fetched[1], KS,
+                   KS / 2);
+      return 12;
+    }
+    std::vector<int32_t> slot_tok(KS);
+    std::vector<uint16_t> staged((size_t)KS * row_bytes / 2);
+    HIP_OK(hipMemcpy(slot_tok.data(), dslot_tok, KS * 4, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(staged.data(), dstaged, staged.size() * 2, hipMemcpyDeviceToHost));
+    std::vector<int32_t> held(slot_tok);
+    std::sort(held.begin(), held.end());
+    std::vector<int32_t> want_b(sel_b);
+    std::sort(want_b.begin(), want_b.end());
+    if (held != want_b) {
+      std::fprintf(stderr, "the staged set is not the second selection\n");
+      return 13;
+    }
+    for (int sl = 0; sl < KS; ++sl)
+      if (std::memcmp(&staged[(size_t)sl * row_bytes / 2], &hsrc[(size_t)slot_tok[sl] * row_bytes / 2], row_bytes) != 0) {
+        std::fprintf(stderr, "slot %d does not hold the row of token %d\n", sl, slot_tok[sl]);
+        return 14;
+      }
+    for (void* p : {dsrc, dstaged, (void*)dsel, (void*)dslot_tok, (void*)dslot_of, (void*)dftok, (void*)dfslot, (void*)dfcount})
+      HIP_OK(hipFree(p));
+  }
 
   HIP_OK(hipStreamDestroy(stream));
   for (void* p : {dk, dv, dq, dout, dws, dgather, (void*)dscores, (void*)didx}) HIP_OK(hipFree(p));
