@@ -153,11 +153,27 @@ def test_argument_validation_happens_before_any_launch():
     # offload staging arguments
     assert lib.okv_offload_stage(None, 4096, fake, 1, fake, 1, fake, None, None) == -1
     assert lib.okv_offload_stage(fake, 4096, fake, 1, fake, 0, fake, None, None) == -1
+    # incremental staging: NULL, too many staged rows, rows that are no multiple of 16 bytes, misaligned buffers
+    assert lib.okv_offload_plan(None, 8, fake, fake, 100, fake, fake, fake, None) == -1
+    assert lib.okv_offload_plan(fake, 0, fake, fake, 100, fake, fake, fake, None) == -1
+    assert lib.okv_offload_plan(fake, (1 << 18) + 1, fake, fake, 1 << 20, fake, fake, fake, None) == -2
+    assert lib.okv_offload_fetch(fake, 4100, fake, fake, fake, 8, fake, None) == -1
+    assert lib.okv_offload_fetch(C.c_void_p(0x1008), 4096, fake, fake, fake, 8, fake, None) == -1
+    assert lib.okv_offload_fetch(fake, 4096, fake, fake, None, 8, fake, None) == -1
+    assert lib.okv_offload_fetch(fake, 4096, fake, fake, fake, 0, fake, None) == 0  # nothing to bound: no launch
+    # the entry point without a workspace refuses what its fixed scratch cannot hold, before anything else
+    assert lib.okv_noalloc_scratch_bytes() == 4 << 20
+    assert lib.okv_sparse_attn_noalloc(fake, fake, fake, C.byref(lay), fake, 40000, None, 40000, None, None, 0, 0, 0,
+                                       None, 0, 64, 1.0, fake, None) == -3
+    assert b"fixed scratch" in lib.okv_last_error()
+    assert lib.okv_sparse_attn_noalloc(fake, fake, fake, None, fake, 8, None, 8, None, None, 0, 0, 0, None, 0, 1, 1.0,
+                                       fake, None) == -1
     # empty work is a successful no-op
     assert lib.okv_topk(fake, 8, None, 0, None, 2, 1, fake, 2, None, 0, None) == 0
     assert lib.okv_score(fake, fake, C.byref(lay), None, 0, 1, 0, 0, 1.0, fake, 0, ws, 1 << 30, None) == 0
     assert lib.okv_set_option(b"no_such_option", 1) == -1
     assert lib.okv_set_option(b"split_rows", 100) == -1
+    assert lib.okv_set_option(b"skip_merge", 1) == -1  # measurement hooks are not options of the public interface
     assert lib.okv_set_option(b"split_rows", 0) == 0
 
 
