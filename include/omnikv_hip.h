@@ -264,6 +264,46 @@ int okv_offload_stage(const void* host_src, int64_t row_bytes, const int32_t* ho
                       void* dev_dst, okv_stream_t copy_stream, void* done_event);
 
 /*
+ * The per-token operations around the attention of a decode step, one launch each.  In the
+ * reference these are third-party module calls (transformers 4.41.2 LlamaRMSNorm,
+ * apply_rotary_pos_emb, LlamaMLP's act_fn(gate) * up) made from the layer forward,
+ * modeling/omnikv.py:155-156 (input_layernorm), :219-227 (self_attn: projections + rotary
+ * embedding), :228-236 (residual add, post_attention_layernorm, mlp); each is a chain of five
+ * to ten elementwise launches there.  All tensors contiguous, same `dtype` (okv_dtype); every
+ * intermediate is rounded to that type where the op-by-op chain rounds it.
+ *   okv_rmsnorm   h = x, or x + residual rounded to dtype and written to sum_out (the new
+ *                 residual stream) when residual != NULL;
+ *                 out = weight * (h * rsqrt(mean(h^2) + eps)) with the normalised h rounded
+ *                 to dtype before the product.  x, residual, sum_out, out: (rows, hidden).
+ *   okv_rope      q_out[r][h] = q[r][h]*cos[r] + rotate_half(q[r][h])*sin[r], the same for k;
+ *                 q row r at q + r*q_row_stride (num_q_heads*head_dim elements, the projection's
+ *                 output), cos / sin (rows, head_dim), q_out (rows, num_q_heads, head_dim),
+ *                 k_out (rows, num_kv_heads, head_dim); head_dim 128.
+ *   okv_rope_append  okv_rope whose rotated k row, and the v row next to it, go straight into a
+ *                 cache's K and V stores: row (request r, kv head h) to
+ *                 store + r*store_batch_stride + h*store_head_stride + pos*store_token_stride
+ *                 (strides in elements), pos = pos_dev[0] (device int64) when pos_dev != NULL.
+ *                 Replaces the rotary embedding and the append of OmniKVMultiStageCache.update
+ *                 for one new token (modeling/spec_cache.py:337-347,358-368).
+ *   okv_silu_mul  out = silu(gate) * up over n elements.
+ */
+int okv_rmsnorm(const void* x, const void* residual, const void* weight, float eps, int32_t rows,
+                int32_t hidden, int32_t dtype, void* sum_out, void* out, okv_stream_t stream);
+int okv_rope(const void* q, int64_t q_row_stride, const void* k, int64_t k_row_stride,
+             const void* cos, const void* sin, int32_t rows, int32_t num_q_heads,
+             int32_t num_kv_heads, int32_t head_dim, int32_t dtype, void* q_out, void* k_out,
+             okv_stream_t stream);
+int okv_rope_append(const void* q, int64_t q_row_stride, const void* k, int64_t k_row_stride,
+                    const void* v, int64_t v_row_stride, const void* cos, const void* sin,
+                    int32_t rows, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                    int32_t dtype, void* q_out, void* k_store, void* v_store,
+                    int64_t store_token_stride, int64_t store_head_stride,
+                    int64_t store_batch_stride, const int64_t* pos_dev, int64_t pos,
+                    okv_stream_t stream);
+int okv_silu_mul(const void* gate, const void* up, int64_t n, int32_t dtype, void* out,
+                 okv_stream_t stream);
+
+/*
  * real_offload tier, incremental.  The rows staged on the device for a group of sparse
  * layers are a set -- attention over them does not depend on their order -- so a new selection
  * keeps the rows it shares with the previous one in place and fetches only the others, into

@@ -34,6 +34,10 @@ EXPORTS = (
     "okv_offload_stage",
     "okv_offload_plan",
     "okv_offload_fetch",
+    "okv_rmsnorm",
+    "okv_rope",
+    "okv_rope_append",
+    "okv_silu_mul",
 )
 
 
@@ -113,6 +117,15 @@ def _declare(l):
     l.okv_offload_plan.argtypes = [vp, i32, vp, vp, i32, vp, vp, vp, vp]
     l.okv_offload_fetch.restype = C.c_int
     l.okv_offload_fetch.argtypes = [vp, i64, vp, vp, vp, i32, vp, vp]
+    l.okv_rmsnorm.restype = C.c_int
+    l.okv_rmsnorm.argtypes = [vp, vp, vp, f32, i32, i32, i32, vp, vp, vp]
+    l.okv_rope.restype = C.c_int
+    l.okv_rope.argtypes = [vp, i64, vp, i64, vp, vp, i32, i32, i32, i32, i32, vp, vp, vp]
+    l.okv_rope_append.restype = C.c_int
+    l.okv_rope_append.argtypes = [vp, i64, vp, i64, vp, i64, vp, vp, i32, i32, i32, i32, i32, vp, vp, vp, i64, i64, i64,
+                                  vp, i64, vp]
+    l.okv_silu_mul.restype = C.c_int
+    l.okv_silu_mul.argtypes = [vp, vp, i64, i32, vp, vp]
     l.okv_offload_stage.restype = C.c_int
     l.okv_offload_stage.argtypes = [vp, i64, vp, i32, vp, i32, vp, vp, vp]
 

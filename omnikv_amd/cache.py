@@ -302,6 +302,20 @@ class OmniKVMultiStageCache:
         st.append(key_states, value_states)
         self._sync_lists(layer_idx)
 
+    def append_projected(self, q_lin: torch.Tensor, k_lin: torch.Tensor, v_lin: torch.Tensor, cos: torch.Tensor,
+                         sin: torch.Tensor, layer_idx: int, num_q_heads: int) -> torch.Tensor:
+        """Static decode: the rotary embedding of the new token's q and k and the append of its k and v rows
+        in one launch (what append() stores, written by the kernel that rotates).  q_lin / k_lin / v_lin are the
+        projections' outputs (bsz, 1, heads * D); returns the rotated q (bsz, Hq, 1, D)."""
+        if not self._static:
+            raise RuntimeError("append_projected serves static decode; elsewhere rotate, then append()")
+        if layer_idx == 0:
+            self._seen_tokens += 1
+        sparse = self.layer_state[layer_idx][0]
+        st = self._tail[layer_idx] if sparse else self._store[layer_idx]
+        return ops.rope_append(q_lin, k_lin, v_lin, cos, sin, num_q_heads, st.k.shape[1], st.k, st.v,
+                               self._tail_pos if sparse else self._pos)
+
     def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int,
                cache_kwargs: Optional[Dict[str, Any]] = None) -> Tuple[torch.Tensor, torch.Tensor]:
         """modeling/spec_cache.py:308-369: store the new rows and return what this

@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
 OUT = os.path.join(PKG, "libomnikv_hip.so")
 SOURCES = ["okv_api.hip", "okv_attn.hip", "okv_attn_mfma.hip", "okv_topk.hip", "okv_topk_mb.hip", "okv_gather.hip",
-           "okv_window.hip", "okv_diag.hip"]
+           "okv_window.hip", "okv_diag.hip", "okv_layer.hip"]
 FLAGS = [
     "--offload-arch=gfx950",
     "-O3",

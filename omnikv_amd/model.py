@@ -16,7 +16,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from . import trace
+from . import ops, trace
 from .cache import OmniKVMultiStageCache, get_cache_cls
 from .config import OmniKVConfig
 from .selector import apply_rotary_pos_emb, select_from_query
@@ -35,17 +35,35 @@ class LlamaShape:
     rms_norm_eps: float = 1e-5
 
 
+# The per-token operations of a decode step (RMSNorm with the residual add in front of it, rotary
+# embedding, SiLU(gate) * up) as one HIP launch each instead of torch's op-by-op chains; prefill and
+# CPU tensors take the torch path.  Off: every op as the reference's modules issue it.
+FUSED_LAYER_OPS = True
+
+
+def _fusable(x: torch.Tensor, *others: torch.Tensor) -> bool:
+    return (FUSED_LAYER_OPS and x.is_cuda and x.shape[-2] == 1 and x.is_contiguous()
+            and all(o.dtype == x.dtype and o.is_contiguous() for o in others))
+
+
 class RMSNorm(nn.Module):
     def __init__(self, dim: int, eps: float):
         super().__init__()
         self.weight = nn.Parameter(torch.ones(dim))
         self.eps = eps
 
-    def forward(self, x):
+    def forward(self, x, residual=None):
+        """Normalised x, or with `residual`: (normalised (x + residual), x + residual)."""
+        if _fusable(x, self.weight, *([residual] if residual is not None else [])):
+            return ops.rmsnorm(x, self.weight, self.eps, residual)
+        total = None
+        if residual is not None:
+            x = total = residual + x
         dt = x.dtype
         x = x.float()
         x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.eps)
-        return self.weight * x.to(dt)
+        x = self.weight * x.to(dt)
+        return x if residual is None else (x, total)
 
 
 class RotaryEmbedding(nn.Module):
@@ -69,7 +87,10 @@ class MLP(nn.Module):
         self.down_proj = nn.Linear(s.intermediate_size, s.hidden_size, bias=False)
 
     def forward(self, x):
-        return self.down_proj(F.silu(self.gate_proj(x)) * self.up_proj(x))
+        gate, up = self.gate_proj(x), self.up_proj(x)
+        if _fusable(gate, up):
+            return self.down_proj(ops.silu_mul(gate, up))
+        return self.down_proj(F.silu(gate) * up)
 
 
 class OmniKVAttention(nn.Module):
@@ -89,14 +110,31 @@ class OmniKVAttention(nn.Module):
         self.o_proj = nn.Linear(self.num_heads * self.head_dim, s.hidden_size, bias=False)
         self.rotary_emb = RotaryEmbedding(self.head_dim, s.rope_theta)
 
-    def qkv(self, hidden_states, position_ids):
+    def qkv(self, hidden_states, position_ids, rope=None):
+        """Rotated q, k and v as (bsz, heads, n, D).  rope: (cos, sin) of these positions when the
+        caller has them already (they are the same for every layer of a step)."""
         b, n, _ = hidden_states.shape
-        q = self.q_proj(hidden_states).view(b, n, self.num_heads, self.head_dim).transpose(1, 2)
-        k = self.k_proj(hidden_states).view(b, n, self.num_key_value_heads, self.head_dim).transpose(1, 2)
-        v = self.v_proj(hidden_states).view(b, n, self.num_key_value_heads, self.head_dim).transpose(1, 2)
-        cos, sin = self.rotary_emb(v, position_ids)
+        q, k, v = self.q_proj(hidden_states), self.k_proj(hidden_states), self.v_proj(hidden_states)
+        v = v.view(b, n, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+        cos, sin = rope if rope is not None else self.rotary_emb(v, position_ids)
+        if n == 1 and self.head_dim == 128 and _fusable(q, k, cos, sin):
+            q, k = ops.rope(q, k, cos, sin, self.num_heads, self.num_key_value_heads)
+            return q, k, v
+        q = q.view(b, n, self.num_heads, self.head_dim).transpose(1, 2)
+        k = k.view(b, n, self.num_key_value_heads, self.head_dim).transpose(1, 2)
         q, k = apply_rotary_pos_emb(q, k, cos, sin)
         return q, k, v
+
+
+    def q_and_append(self, hidden_states, position_ids, rope, cache):
+        """One new token: the rotated q (bsz, Hq, 1, D), with the rotated k and the v appended to the cache."""
+        if getattr(cache, "_static", False) and self.head_dim == 128 and rope is not None:
+            q, k, v = self.q_proj(hidden_states), self.k_proj(hidden_states), self.v_proj(hidden_states)
+            if _fusable(q, k, v, rope[0], rope[1]):  # rotation and append in one launch
+                return cache.append_projected(q, k, v, rope[0], rope[1], self.layer_idx, self.num_heads)
+        q, k, v = self.qkv(hidden_states, position_ids, rope)
+        cache.append(k, v, self.layer_idx)
+        return q
 
 
 class OmniKVMulLayer(nn.Module):
@@ -118,9 +156,15 @@ class OmniKVMulLayer(nn.Module):
         self.window_size = config.get("window_size", 16)
         self.decode_step = 0
 
-    def forward(self, hidden_states, position_ids, past_key_value: OmniKVMultiStageCache):
-        residual = hidden_states
-        hidden_states = self.input_layernorm(hidden_states)
+    def forward(self, hidden_states, position_ids, past_key_value: OmniKVMultiStageCache, delta=None, rope=None,
+                defer_add: bool = False):
+        """delta: what the previous layer left to be added to hidden_states (its MLP output), folded
+        into this layer's first norm; defer_add: return (hidden_states, mlp output) instead of their sum."""
+        if delta is not None:
+            hidden_states, residual = self.input_layernorm(delta, residual=hidden_states)
+        else:
+            residual = hidden_states
+            hidden_states = self.input_layernorm(hidden_states)
         q_len = hidden_states.shape[1]
         if q_len > 1:
             self.prefill_len = q_len
@@ -129,8 +173,8 @@ class OmniKVMulLayer(nn.Module):
                 self.decode_step = 1
         assert isinstance(past_key_value, self.cache_cls)
         attn = self.self_attn
-        q, k, v = attn.qkv(hidden_states, position_ids)
         if q_len > 1:
+            q, k, v = attn.qkv(hidden_states, position_ids, rope)
             # prefill: store K/V (tiered by the cache), causal attention over the prompt
             past_key_value.append(k, v, self.layer_idx)
             out = F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
@@ -140,7 +184,7 @@ class OmniKVMulLayer(nn.Module):
             num_selected_tokens = self.config.get("num_of_selected_tokens", 4096)
             if isinstance(num_selected_tokens, float):
                 num_selected_tokens = int(num_selected_tokens * consider_len)
-            past_key_value.append(k, v, self.layer_idx)
+            q = attn.q_and_append(hidden_states, position_ids, rope, past_key_value)
             if trace.idx_tracer is not None:
                 # every layer reports what it would select (modeling/offload_select_once.py:170-174)
                 trace.idx_tracer.observe(self.layer_idx, q, past_key_value.key_cache[self.layer_idx], consider_len)
@@ -173,10 +217,13 @@ class OmniKVMulLayer(nn.Module):
             else:
                 o = past_key_value.attend(q, self.layer_idx)
             out = o.reshape(hidden_states.shape[0], 1, -1)
-        hidden_states = residual + attn.o_proj(out)
-        residual = hidden_states
-        hidden_states = self.post_attention_layernorm(hidden_states)
-        hidden_states = torch.cat([self.mlp(hs) for hs in torch.split(hidden_states, 4000, dim=1)], dim=1)
+        hidden_states, residual = self.post_attention_layernorm(attn.o_proj(out), residual=residual)
+        if hidden_states.shape[1] <= 4000:
+            hidden_states = self.mlp(hidden_states)
+        else:  # modeling/omnikv.py:233-235: long prompts go through the MLP in pieces
+            hidden_states = torch.cat([self.mlp(hs) for hs in torch.split(hidden_states, 4000, dim=1)], dim=1)
+        if defer_add:
+            return residual, hidden_states
         return residual + hidden_states
 
 
@@ -189,9 +236,18 @@ class OmniKVMulModel(nn.Module):
 
     def forward(self, input_ids, position_ids, past_key_values):
         h = self.embed_tokens(input_ids)
+        if input_ids.shape[1] > 1 or not FUSED_LAYER_OPS or not h.is_cuda:
+            for layer in self.layers:
+                h = layer(h, position_ids, past_key_values)
+            return self.norm(h)
+        # decode: cos / sin of the position once for all layers; every layer's closing residual add is
+        # folded into the norm that follows it
+        attn0 = self.layers[0].self_attn
+        rope = attn0.rotary_emb(h, position_ids)
+        delta = None
         for layer in self.layers:
-            h = layer(h, position_ids, past_key_values)
-        return self.norm(h)
+            h, delta = layer(h, position_ids, past_key_values, delta=delta, rope=rope, defer_add=True)
+        return self.norm(delta, residual=h)[0]
 
 
 class StaticDecodeGraph:

@@ -342,3 +342,79 @@ def gather_rows(src, idx: torch.Tensor, out: Optional[torch.Tensor] = None,
         sp, C.byref(lay), idx.data_ptr(), idx.stride(0), _lens(sel_lens, batch, "sel_lens"), ksel,
         batch, out.data_ptr(), out.stride(2), out.stride(1), out.stride(0), _stream_ptr(idx.device)))
     return out
+
+
+# ---------------------------------------------------------------- per-token layer operations
+def _same(*ts):
+    t0 = ts[0]
+    for t in ts:
+        _require_gpu(t, "tensor")
+        if t.dtype != t0.dtype or not t.is_contiguous():
+            raise ValueError("operands must be contiguous GPU tensors of one dtype")
+    if t0.dtype not in _DTYPES:
+        raise ValueError("dtype must be float32, bfloat16 or float16")
+    return _DTYPES[t0.dtype]
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: Optional[torch.Tensor] = None):
+    """weight * rms_normalise(x [+ residual]) over the last dimension; okv_rmsnorm.  Returns the
+    normalised tensor, or (normalised, x + residual) when a residual is given."""
+    dt = _same(x, weight) if residual is None else _same(x, weight, residual)
+    hidden = x.shape[-1]
+    rows = x.numel() // hidden
+    out = torch.empty_like(x)
+    total = torch.empty_like(x) if residual is not None else None
+    check(lib().okv_rmsnorm(x.data_ptr(), residual.data_ptr() if residual is not None else None, weight.data_ptr(),
+                            float(eps), rows, hidden, dt, total.data_ptr() if total is not None else None,
+                            out.data_ptr(), _stream_ptr(x.device)))
+    return out if residual is None else (out, total)
+
+
+def rope(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, num_q_heads: int,
+         num_kv_heads: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Rotary embedding of one position per request: q (bsz, 1, Hq*D) and k (bsz, 1, Hkv*D) as the
+    projections leave them, cos / sin (bsz, 1, D); returns (bsz, Hq, 1, D) and (bsz, Hkv, 1, D).  okv_rope."""
+    dt = _same(q, k, cos, sin)
+    bsz = q.shape[0]
+    d = cos.shape[-1]
+    if q.shape[1] != 1 or q.shape[-1] != num_q_heads * d or k.shape[-1] != num_kv_heads * d:
+        raise ValueError("q / k must be (bsz, 1, heads * head_dim)")
+    q_out = torch.empty((bsz, num_q_heads, 1, d), dtype=q.dtype, device=q.device)
+    k_out = torch.empty((bsz, num_kv_heads, 1, d), dtype=q.dtype, device=q.device)
+    check(lib().okv_rope(q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), cos.data_ptr(), sin.data_ptr(), bsz,
+                         num_q_heads, num_kv_heads, d, dt, q_out.data_ptr(), k_out.data_ptr(), _stream_ptr(q.device)))
+    return q_out, k_out
+
+
+def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                num_q_heads: int, num_kv_heads: int, k_store: torch.Tensor, v_store: torch.Tensor,
+                pos) -> torch.Tensor:
+    """`rope` whose rotated k row and the v row are written into k_store / v_store (bsz, Hkv, capacity, D) at
+    token position `pos` (an int, or a one-element int64 GPU tensor read by the kernel); returns the rotated
+    q (bsz, Hq, 1, D).  okv_rope_append."""
+    dt = _same(q, k, v, cos, sin)
+    bsz, d = q.shape[0], cos.shape[-1]
+    if k_store.dtype != q.dtype or k_store.stride() != v_store.stride() or k_store.stride(-1) != 1:
+        raise ValueError("k_store / v_store must share dtype with q and strides with each other")
+    if k_store.shape[0] != bsz or k_store.shape[1] != num_kv_heads or k_store.shape[3] != d:
+        raise ValueError("stores must be (bsz, Hkv, capacity, D)")
+    q_out = torch.empty((bsz, num_q_heads, 1, d), dtype=q.dtype, device=q.device)
+    on_dev = isinstance(pos, torch.Tensor)
+    if on_dev and (pos.dtype != torch.int64 or not pos.is_cuda or pos.numel() != 1):
+        raise ValueError("a device position must be a one-element int64 GPU tensor")
+    if not on_dev and not 0 <= int(pos) < k_store.shape[2]:
+        raise ValueError("position outside the store")
+    check(lib().okv_rope_append(q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
+                                cos.data_ptr(), sin.data_ptr(), bsz, num_q_heads, num_kv_heads, d, dt, q_out.data_ptr(),
+                                k_store.data_ptr(), v_store.data_ptr(), k_store.stride(2), k_store.stride(1),
+                                k_store.stride(0), pos.data_ptr() if on_dev else None, 0 if on_dev else int(pos),
+                                _stream_ptr(q.device)))
+    return q_out
+
+
+def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """silu(gate) * up; okv_silu_mul."""
+    dt = _same(gate, up)
+    out = torch.empty_like(gate)
+    check(lib().okv_silu_mul(gate.data_ptr(), up.data_ptr(), gate.numel(), dt, out.data_ptr(), _stream_ptr(gate.device)))
+    return out
