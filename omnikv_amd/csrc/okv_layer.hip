@@ -34,24 +34,63 @@ __device__ __forceinline__ float rnd(float v) {
 template <>
 __device__ __forceinline__ float rnd<float>(float v) { return v; }
 
-// grid (rows), 256 threads.  h = x (+ residual, rounded to T and written to sum_out when asked for);
-// out = T(weight * T(h * rsqrt(mean(h^2) + eps))).
+// Eight consecutive elements of type T as fp32 (one 16- or 32-byte load) and back.
 template <typename T>
+__device__ __forceinline__ void ld8(const T* p, float (&o)[8]) { load8(p, o); }
+template <typename T>
+__device__ __forceinline__ void st8(T* p, const float (&v)[8]) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) store1(p + i, v[i]);
+}
+
+// grid (rows), 256 threads.  h = x (+ residual, rounded to T and written to sum_out when asked for);
+// out = T(weight * T(h * rsqrt(mean(h^2) + eps))).  A thread owns up to CH chunks of eight consecutive
+// elements and keeps them in registers between the two passes, every load of a pass in flight at once
+// (one launch, a handful of rows: the time is the length of the dependent chain, not the bytes);
+// rows longer than 256 * 8 * CH elements, or not a multiple of eight, take the element-wise loop.
+template <typename T, int CH>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ residual,
                                                       const T* __restrict__ weight, float eps, int hidden,
-                                                      T* __restrict__ sum_out, T* __restrict__ out) {
+                                                      int aligned16, T* __restrict__ sum_out, T* __restrict__ out) {
   __shared__ float part[4];
   const int64_t row = blockIdx.x;
   const T* xr = x + row * hidden;
   const T* rr = residual ? residual + row * hidden : nullptr;
+  const bool vec = aligned16 && (hidden & 7) == 0 && hidden <= 256 * 8 * CH;
+  float h[CH][8];
   float ss = 0.f;
-  for (int i = threadIdx.x; i < hidden; i += 256) {
-    float h = ld1<T>(xr + i);
-    if (rr) {
-      h = rnd<T>(h + ld1<T>(rr + i));
-      store1(sum_out + row * hidden + i, h);
+  if (vec) {
+    float r[CH][8];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int i = (c * 256 + (int)threadIdx.x) * 8;
+      if (i < hidden) {
+        ld8<T>(xr + i, h[c]);
+        if (rr) ld8<T>(rr + i, r[c]);
+      }
     }
-    ss = fmaf(h, h, ss);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int i = (c * 256 + (int)threadIdx.x) * 8;
+      if (i < hidden) {
+        if (rr) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) h[c][e] = rnd<T>(h[c][e] + r[c][e]);
+          st8<T>(sum_out + row * hidden + i, h[c]);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss = fmaf(h[c][e], h[c][e], ss);
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += 256) {
+      float v = ld1<T>(xr + i);
+      if (rr) {
+        v = rnd<T>(v + ld1<T>(rr + i));
+        store1(sum_out + row * hidden + i, v);
+      }
+      ss = fmaf(v, v, ss);
+    }
   }
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) ss += __shfl_xor(ss, o);
@@ -59,9 +98,23 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const T* __restrict__ x, c
   __syncthreads();
   const float var = ((part[0] + part[1]) + (part[2] + part[3])) / (float)hidden;
   const float rstd = rsqrtf(var + eps);
-  const T* hr = rr ? sum_out + row * hidden : xr;  // this thread re-reads what it wrote itself
-  for (int i = threadIdx.x; i < hidden; i += 256)
-    store1(out + row * hidden + i, ld1<T>(weight + i) * rnd<T>(ld1<T>(hr + i) * rstd));
+  if (vec) {
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int i = (c * 256 + (int)threadIdx.x) * 8;
+      if (i < hidden) {
+        float w[8], o[8];
+        ld8<T>(weight + i, w);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = w[e] * rnd<T>(h[c][e] * rstd);
+        st8<T>(out + row * hidden + i, o);
+      }
+    }
+  } else {
+    const T* hr = rr ? sum_out + row * hidden : xr;  // this thread re-reads what it wrote itself
+    for (int i = threadIdx.x; i < hidden; i += 256)
+      store1(out + row * hidden + i, ld1<T>(weight + i) * rnd<T>(ld1<T>(hr + i) * rstd));
+  }
 }
 
 // grid (rows, heads_q + heads_k [+ heads_k]), 64 threads (D = 128: a lane owns elements l and l + 64).
@@ -101,21 +154,34 @@ __global__ __launch_bounds__(64) void rope_kernel(const T* __restrict__ q, const
   store1(dst + l + 64, rnd<T>(x1 * c1) + rnd<T>(x0 * s1));
 }
 
-// out = T(T(silu(gate)) * up), silu(g) = g / (1 + exp(-g)); 8 elements per thread.
-template <typename T>
+// out = T(T(silu(gate)) * up), silu(g) = g / (1 + exp(-g)); eight consecutive elements per thread
+// (n a multiple of 8 and 16-byte aligned operands), else one.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ gate, const T* __restrict__ up,
                                                        int64_t n, T* __restrict__ out) {
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
-    const float g = ld1<T>(gate + i);
-    store1(out + i, rnd<T>(g / (1.0f + expf(-g))) * ld1<T>(up + i));
+  if (VEC) {
+    for (int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8; i < n; i += (int64_t)gridDim.x * 256 * 8) {
+      float g[8], u[8], o[8];
+      ld8<T>(gate + i, g);
+      ld8<T>(up + i, u);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = rnd<T>(g[e] / (1.0f + expf(-g[e]))) * u[e];
+      st8<T>(out + i, o);
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+      const float g = ld1<T>(gate + i);
+      store1(out + i, rnd<T>(g / (1.0f + expf(-g))) * ld1<T>(up + i));
+    }
   }
 }
 
 template <typename T>
 static void launch_rmsnorm(const void* x, const void* residual, const void* weight, float eps, int rows, int hidden,
                            void* sum_out, void* out, hipStream_t stream) {
-  hipLaunchKernelGGL(rmsnorm_kernel<T>, dim3(rows), dim3(256), 0, stream, (const T*)x, (const T*)residual,
-                     (const T*)weight, eps, hidden, (T*)sum_out, (T*)out);
+  const uintptr_t all = (uintptr_t)x | (uintptr_t)residual | (uintptr_t)weight | (uintptr_t)sum_out | (uintptr_t)out;
+  hipLaunchKernelGGL((rmsnorm_kernel<T, 4>), dim3(rows), dim3(256), 0, stream, (const T*)x, (const T*)residual,
+                     (const T*)weight, eps, hidden, (int)((all & 15) == 0), (T*)sum_out, (T*)out);
 }
 template <typename T>
 static void launch_rope(const void* q, const void* k, const void* v, const void* cos, const void* sin, int rows,
@@ -128,10 +194,15 @@ static void launch_rope(const void* q, const void* k, const void* v, const void*
 }
 template <typename T>
 static void launch_silu_mul(const void* gate, const void* up, int64_t n, void* out, hipStream_t stream) {
-  int64_t blocks = (n + 255) / 256;
+  const bool vec = n % 8 == 0 && (((uintptr_t)gate | (uintptr_t)up | (uintptr_t)out) & 15) == 0;
+  int64_t blocks = ((vec ? n / 8 : n) + 255) / 256;
   if (blocks > 4096) blocks = 4096;
-  hipLaunchKernelGGL(silu_mul_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, (const T*)gate, (const T*)up,
-                     n, (T*)out);
+  if (vec)
+    hipLaunchKernelGGL((silu_mul_kernel<T, true>), dim3((unsigned)blocks), dim3(256), 0, stream, (const T*)gate,
+                       (const T*)up, n, (T*)out);
+  else
+    hipLaunchKernelGGL((silu_mul_kernel<T, false>), dim3((unsigned)blocks), dim3(256), 0, stream, (const T*)gate,
+                       (const T*)up, n, (T*)out);
 }
 
 }  // namespace okv
