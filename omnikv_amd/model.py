@@ -79,15 +79,35 @@ class RotaryEmbedding(nn.Module):
         return emb.cos().to(x.dtype), emb.sin().to(x.dtype)
 
 
+class _Rows:
+    """A block of output rows of a merged projection, usable like the nn.Linear it stands for: `.weight` is a
+    view of the merged weight, calling it multiplies by those rows only.  The merged module owns the parameter
+    (q/k/v share one GEMM per token, gate/up another: at batch 1 a projection is a memory-bound GEMV and the
+    small ones are pure launch latency); code written against q_proj / k_proj / ... keeps working."""
+
+    def __init__(self, linear: nn.Linear, lo: int, hi: int):
+        self.linear, self.lo, self.hi = linear, lo, hi
+
+    @property
+    def weight(self):
+        return self.linear.weight[self.lo: self.hi]
+
+    def __call__(self, x):
+        return F.linear(x, self.weight)
+
+
 class MLP(nn.Module):
     def __init__(self, s: LlamaShape):
         super().__init__()
-        self.gate_proj = nn.Linear(s.hidden_size, s.intermediate_size, bias=False)
-        self.up_proj = nn.Linear(s.hidden_size, s.intermediate_size, bias=False)
+        self.inter = s.intermediate_size
+        self.gate_up_proj = nn.Linear(s.hidden_size, 2 * s.intermediate_size, bias=False)  # rows: gate, then up
+        self.gate_proj = _Rows(self.gate_up_proj, 0, self.inter)
+        self.up_proj = _Rows(self.gate_up_proj, self.inter, 2 * self.inter)
         self.down_proj = nn.Linear(s.intermediate_size, s.hidden_size, bias=False)
 
     def forward(self, x):
-        gate, up = self.gate_proj(x), self.up_proj(x)
+        gu = self.gate_up_proj(x)
+        gate, up = gu[..., : self.inter], gu[..., self.inter:]
         if _fusable(gate, up):
             return self.down_proj(ops.silu_mul(gate, up))
         return self.down_proj(F.silu(gate) * up)
@@ -104,17 +124,25 @@ class OmniKVAttention(nn.Module):
         self.num_key_value_heads = s.num_key_value_heads
         self.num_key_value_groups = self.num_heads // self.num_key_value_heads
         self.head_dim = s.head_dim
-        self.q_proj = nn.Linear(s.hidden_size, self.num_heads * self.head_dim, bias=False)
-        self.k_proj = nn.Linear(s.hidden_size, self.num_key_value_heads * self.head_dim, bias=False)
-        self.v_proj = nn.Linear(s.hidden_size, self.num_key_value_heads * self.head_dim, bias=False)
+        nq, nkv = self.num_heads * self.head_dim, self.num_key_value_heads * self.head_dim
+        self.qkv_proj = nn.Linear(s.hidden_size, nq + 2 * nkv, bias=False)  # rows: q, then k, then v
+        self.q_proj = _Rows(self.qkv_proj, 0, nq)
+        self.k_proj = _Rows(self.qkv_proj, nq, nq + nkv)
+        self.v_proj = _Rows(self.qkv_proj, nq + nkv, nq + 2 * nkv)
         self.o_proj = nn.Linear(self.num_heads * self.head_dim, s.hidden_size, bias=False)
         self.rotary_emb = RotaryEmbedding(self.head_dim, s.rope_theta)
+
+    def _project(self, hidden_states):
+        """q, k, v of one merged GEMM, as views (bsz, n, heads * D) of its output."""
+        nq, nkv = self.num_heads * self.head_dim, self.num_key_value_heads * self.head_dim
+        qkv = self.qkv_proj(hidden_states)
+        return qkv[..., :nq], qkv[..., nq: nq + nkv], qkv[..., nq + nkv:]
 
     def qkv(self, hidden_states, position_ids, rope=None):
         """Rotated q, k and v as (bsz, heads, n, D).  rope: (cos, sin) of these positions when the
         caller has them already (they are the same for every layer of a step)."""
         b, n, _ = hidden_states.shape
-        q, k, v = self.q_proj(hidden_states), self.k_proj(hidden_states), self.v_proj(hidden_states)
+        q, k, v = self._project(hidden_states)
         v = v.view(b, n, self.num_key_value_heads, self.head_dim).transpose(1, 2)
         cos, sin = rope if rope is not None else self.rotary_emb(v, position_ids)
         if n == 1 and self.head_dim == 128 and _fusable(q, k, cos, sin):
@@ -129,7 +157,7 @@ class OmniKVAttention(nn.Module):
     def q_and_append(self, hidden_states, position_ids, rope, cache):
         """One new token: the rotated q (bsz, Hq, 1, D), with the rotated k and the v appended to the cache."""
         if getattr(cache, "_static", False) and self.head_dim == 128 and rope is not None:
-            q, k, v = self.q_proj(hidden_states), self.k_proj(hidden_states), self.v_proj(hidden_states)
+            q, k, v = self._project(hidden_states)
             if _fusable(q, k, v, rope[0], rope[1]):  # rotation and append in one launch
                 return cache.append_projected(q, k, v, rope[0], rope[1], self.layer_idx, self.num_heads)
         q, k, v = self.qkv(hidden_states, position_ids, rope)
@@ -283,6 +311,39 @@ class OmniKVMulLM(nn.Module):
             if p.dim() >= 2:
                 p.normal_(0.0, std, generator=g)
         return self
+
+    @torch.no_grad()
+    def load_llama_state_dict(self, state_dict) -> None:
+        """Weights under the names a Llama checkpoint uses (the reference loads one with from_pretrained,
+        infer.py): `...self_attn.{q,k,v}_proj.weight` go into the rows of the merged `qkv_proj.weight`,
+        `...mlp.{gate,up}_proj.weight` into `gate_up_proj.weight`, everything else by its own name."""
+        own = dict(self.named_parameters())
+        seen = set()
+        for name, w in state_dict.items():
+            parts = name.rsplit(".", 2)
+            if len(parts) == 3 and parts[2] == "weight" and parts[1] in ("q_proj", "k_proj", "v_proj", "gate_proj", "up_proj"):
+                merged = "qkv_proj" if parts[1][0] in "qkv" else "gate_up_proj"
+                mod = self.get_submodule(parts[0])
+                rows = getattr(mod, parts[1])
+                dst = own[f"{parts[0]}.{merged}.weight"][rows.lo: rows.hi]
+                if dst.shape != w.shape:
+                    raise ValueError(f"{name}: shape {tuple(w.shape)}, expected {tuple(dst.shape)}")
+                dst.copy_(w)
+                seen.add((parts[0], parts[1]))
+            elif name in own:
+                if own[name].shape != w.shape:
+                    raise ValueError(f"{name}: shape {tuple(w.shape)}, expected {tuple(own[name].shape)}")
+                own[name].copy_(w)
+                seen.add(name)
+            elif not name.endswith("rotary_emb.inv_freq"):
+                raise KeyError(f"unexpected key {name}")
+        missing = [n for n in own if n not in seen and not n.endswith(("qkv_proj.weight", "gate_up_proj.weight"))]
+        for li in range(self.shape.num_hidden_layers):
+            for mod, names in ((f"model.layers.{li}.self_attn", ("q_proj", "k_proj", "v_proj")),
+                               (f"model.layers.{li}.mlp", ("gate_proj", "up_proj"))):
+                missing += [f"{mod}.{n}.weight" for n in names if (mod, n) not in seen]
+        if missing:
+            raise KeyError(f"missing keys: {missing[:5]}{' ...' if len(missing) > 5 else ''}")
 
     def new_cache(self, **kwargs) -> OmniKVMultiStageCache:
         sel = [int(i) for i in self.config.get("do_select_layers").split(",")]

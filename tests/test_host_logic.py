@@ -292,3 +292,49 @@ def test_static_decode_budget_is_counted_on_the_host():
     assert g.graph.replays == 2  # the refused replay launched nothing
     with pytest.raises(RuntimeError):
         c.note_static_step()
+
+
+def test_llama_checkpoint_names_load_into_the_merged_projections():
+    """q/k/v and gate/up share one weight each here; a state dict with the per-projection names of a Llama
+    checkpoint fills the right rows, and the per-projection handles keep computing what separate layers would."""
+    from omnikv_amd.model import LlamaShape, OmniKVMulLM
+
+    shape = LlamaShape(hidden_size=256, intermediate_size=384, vocab_size=100, num_hidden_layers=2,
+                       num_attention_heads=4, num_key_value_heads=2, head_dim=128)
+    cfg = okv_config.OmniKVConfig(model_cls="multi", cache_cls="multi", do_select_layers="0", num_wait_load_layers=1,
+                                  real_offload=False, dense_more=True, num_of_selected_tokens=0.5, selector_cls="last")
+    lm = OmniKVMulLM(shape, cfg).float()
+    g = torch.Generator().manual_seed(0)
+    sd = {"model.embed_tokens.weight": torch.randn(100, 256, generator=g), "model.norm.weight": torch.randn(256, generator=g),
+          "lm_head.weight": torch.randn(100, 256, generator=g)}
+    for li in range(2):
+        p = f"model.layers.{li}."
+        sd.update({p + "self_attn.q_proj.weight": torch.randn(512, 256, generator=g),
+                   p + "self_attn.k_proj.weight": torch.randn(256, 256, generator=g),
+                   p + "self_attn.v_proj.weight": torch.randn(256, 256, generator=g),
+                   p + "self_attn.o_proj.weight": torch.randn(256, 512, generator=g),
+                   p + "mlp.gate_proj.weight": torch.randn(384, 256, generator=g),
+                   p + "mlp.up_proj.weight": torch.randn(384, 256, generator=g),
+                   p + "mlp.down_proj.weight": torch.randn(256, 384, generator=g),
+                   p + "input_layernorm.weight": torch.randn(256, generator=g),
+                   p + "post_attention_layernorm.weight": torch.randn(256, generator=g),
+                   p + "self_attn.rotary_emb.inv_freq": torch.zeros(64)})
+    lm.load_llama_state_dict(sd)
+    x = torch.randn(1, 3, 256, generator=g)
+    for li in range(2):
+        a, m = lm.model.layers[li].self_attn, lm.model.layers[li].mlp
+        p = f"model.layers.{li}."
+        for name in ("q_proj", "k_proj", "v_proj"):
+            assert torch.equal(getattr(a, name).weight, sd[p + f"self_attn.{name}.weight"])
+            assert torch.allclose(getattr(a, name)(x), x @ sd[p + f"self_attn.{name}.weight"].T, atol=1e-5)
+        q, k, v = a._project(x)
+        assert torch.allclose(k, x @ sd[p + "self_attn.k_proj.weight"].T, atol=1e-4)
+        want = (torch.nn.functional.silu(x @ sd[p + "mlp.gate_proj.weight"].T) * (x @ sd[p + "mlp.up_proj.weight"].T)) \
+            @ sd[p + "mlp.down_proj.weight"].T
+        assert torch.allclose(m(x), want, atol=1e-3)
+    del sd["model.layers.1.mlp.up_proj.weight"]
+    with pytest.raises(KeyError, match="missing"):
+        lm.load_llama_state_dict(sd)
+    sd["model.layers.1.mlp.up_proj.weight"] = torch.zeros(3, 3)
+    with pytest.raises(ValueError, match="shape"):
+        lm.load_llama_state_dict(sd)
