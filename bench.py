@@ -133,6 +133,57 @@ def make_step(ks, vs, qs, n, tail, k_sel, selector, overlap_select=False):
     return step
 
 
+def cpu_baseline(n, k_sel, selector, budget_s=25.0):
+    """The CPU oracle on this host: one dense layer, one filter layer (score +
+    top-k + dense attention) and one sparse layer (gather + cat + attention) at
+    the benchmark's context length in fp32, scaled to the 32-layer schedule."""
+    from omnikv_amd import synth
+    from oracle import okv_oracle as orc
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    q, k, v = synth.filter_layer_inputs(n, HQ, HKV, D)
+    qn = synth.fresh_q()
+    tk, tv = torch.randn(1, HKV, 1, D), torch.randn(1, HKV, 1, D)
+
+    def t(fn, reps):
+        best = []
+        for _ in range(reps):
+            s = time.perf_counter()
+            r = fn()
+            best.append(time.perf_counter() - s)
+        best.sort()
+        return best[len(best) // 2], r
+
+    t0 = time.perf_counter()
+    dense_s, _ = t(lambda: orc.gqa_attention(q, k, v), 1)
+    reps = 3 if (time.perf_counter() - t0) * 8 < budget_s else 1
+    dense_s, _ = t(lambda: orc.gqa_attention(q, k, v), reps)
+    score_s, sc = t(lambda: orc.score_tokens(q, k, n, selector), reps)
+    topk_s, idx = t(lambda: orc.select_topk(sc, k_sel), reps)
+
+    def sparse():
+        pk = torch.cat([orc.gather_rows(k, idx[0]), tk], dim=-2)
+        pv = torch.cat([orc.gather_rows(v, idx[0]), tv], dim=-2)
+        return orc.gqa_attention(qn, pk, pv)
+
+    sparse_s, _ = t(sparse, max(reps, 3))
+    kinds = schedule()
+    nd = sum(1 for x in kinds.values() if x[0] in ("dense", "filter"))
+    nf = sum(1 for x in kinds.values() if x[0] == "filter")
+    ns = sum(1 for x in kinds.values() if x[0] == "sparse")
+    step_s = nd * dense_s + nf * (score_s + topk_s) + ns * sparse_s
+    return {
+        "value": step_s * 1e6 / LAYERS,
+        "unit": "us/layer",
+        "cores": cores,
+        "kind": "port",
+        "sample": (f"torch fp32 CPU oracle at N={n}: 1 dense layer {dense_s*1e3:.1f} ms, score {score_s*1e3:.1f} ms, "
+                   f"top-k {topk_s*1e3:.2f} ms, 1 sparse layer (gather+cat+attention, k={k_sel}) {sparse_s*1e3:.2f} ms; "
+                   f"median of {reps}; scaled to {nd} dense + {nf} score/top-k + {ns} sparse layers"),
+    }
+
+
 def time_graph(fn, launches, reps, stream):
     """Microseconds per launch of fn()'s `launches` launches: captured once, replayed between two events."""
     fn()
