@@ -113,11 +113,13 @@ def make_step(ks, vs, qs, n, tail, k_sel, selector, overlap_select=False):
             if kind == "dense":
                 outs.append(ops.dense_attn(qs[l], kfull, vfull))
             elif kind == "filter":
-                o, sc = ops.dense_attn(qs[l], kfull, vfull, selector=selector, score_len=n, scores_out=scores[l])
-                outs.append(o)
-                if side is None:
-                    ops.topk(sc, k_sel, out=idx[l])
+                if side is None:  # attention, scores and selection in one call
+                    o, sc, _ = ops.dense_attn(qs[l], kfull, vfull, selector=selector, score_len=n,
+                                              scores_out=scores[l], select_k=k_sel, idx_out=idx[l])
+                    outs.append(o)
                 else:
+                    o, sc = ops.dense_attn(qs[l], kfull, vfull, selector=selector, score_len=n, scores_out=scores[l])
+                    outs.append(o)
                     side.wait_stream(main)
                     with torch.cuda.stream(side):
                         ops.topk(sc, k_sel, out=idx[l])
@@ -280,6 +282,15 @@ def measure_kernels(ops, l, check, stream, ks, vs, qs, n, tail, k_sel, selector,
     sc = ops.score(qs[filter_layers[0]], ks[filter_layers[0]][:, :, :n], selector=selector)
     entry("topk_op", "okv::topk_mb_hist + topk_mb_cand + topk_mb_write (k = %d of %d)" % (k_sel, n),
           time_graph(lambda: [ops.topk(sc, k_sel) for _ in range(4)], 4, reps, stream), None, 3)
+
+    def fused_select():
+        for layer in filter_layers:
+            ops.dense_attn(qs[layer], *full(layer), selector=selector, score_len=n, select_k=k_sel)
+
+    entry("filter_layer_with_selection",
+          "split pass + okv::merge_and_finish + topk_mb_hist + topk_mb_cand + topk_mb_write: "
+          "attention, scores and the k = %d selection of a filter layer in one call" % k_sel,
+          time_graph(fused_select, len(filter_layers), reps, stream), fused_bytes, 5)
 
     def sparse():
         for layer in sparse_layers:

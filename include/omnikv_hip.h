@@ -65,7 +65,8 @@ enum okv_op {
   OKV_OP_TOPK = 1,
   OKV_OP_DENSE_ATTN = 2, /* with or without the fused score output */
   OKV_OP_SPARSE_ATTN = 3,
-  OKV_OP_SCORE_WINDOW = 4
+  OKV_OP_SCORE_WINDOW = 4,
+  OKV_OP_DENSE_ATTN_SELECT = 5
 };
 
 typedef struct okv_kv_layout {
@@ -189,6 +190,25 @@ int okv_dense_attn(const void* q, const void* k_base, const void* v_base,
                    int32_t head_reduce, int32_t normalise, float* scores,
                    int64_t score_stride, void* ws, size_t ws_bytes,
                    okv_stream_t stream);
+
+/*
+ * The whole filter layer in one call: okv_dense_attn with the score output, followed by
+ * okv_topk over those scores (seq_lens = score_lens, max_seq_len = max_score_len), with the
+ * same results as the two calls: out, scores and idx_out are all written, from one workspace.
+ * Replaces the filter layer's selection and the attention that follows it in the same
+ * decoder-layer forward: modeling/omnikv.py:173-216 (select_tokens_by_attn_universal, :8-110,
+ * called at :189-198) and the attention at :219-227; and flash_decode_stage1_with_score +
+ * torch.topk, omnikv-lightllm/.../flash_decoding.py:62-83.
+ * Workspace: okv_workspace_bytes(OKV_OP_DENSE_ATTN_SELECT, ...).
+ */
+int okv_dense_attn_select(const void* q, const void* k_base, const void* v_base,
+                          const okv_kv_layout_t* layout, const int32_t* seq_lens,
+                          int32_t max_seq_len, int32_t batch, float scale, void* out,
+                          const int32_t* score_lens, int32_t max_score_len,
+                          int32_t head_reduce, int32_t normalise, float* scores,
+                          int64_t score_stride, const int32_t* k_per_seg, int32_t max_k,
+                          int32_t* idx_out, int64_t idx_stride, void* ws, size_t ws_bytes,
+                          okv_stream_t stream);
 
 /*
  * Fused gather + sparse GQA decode attention.  Request b attends to the rows

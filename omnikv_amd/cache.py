@@ -624,27 +624,27 @@ class OmniKVMultiStageCache:
 
     def attend_and_select(self, query_states: torch.Tensor, layer_idx: int, num_selected_tokens: int,
                           consider_len: int, selector_cls: str = "last", scale: Optional[float] = None):
-        """Filter layer: dense attention and the filter-layer scores in one pass over
-        K, then top-k and set_idx_on_gpu (modeling/omnikv.py:189-212 followed by the
-        layer's own attention).  Returns (attention output, idx int32 (bsz, k))."""
+        """Filter layer: dense attention, the filter-layer scores from the same pass over K and
+        the top-k of those scores in one library call, then set_idx_on_gpu
+        (modeling/omnikv.py:189-212 followed by the layer's own attention).  Returns
+        (attention output, idx int32 (bsz, k))."""
+        k = min(num_selected_tokens, consider_len)
         if self._static:
             st = self._store[layer_idx]
-            out, scores = ops.dense_attn(query_states, st.k, st.v, seq_len=st.capacity, seq_lens=self._len32,
-                                         selector=selector_cls, score_len=consider_len, scale=scale)
-            k = min(num_selected_tokens, consider_len)
             buf = self._idx.get(layer_idx)
             if buf is None or buf.shape[1] != k:
-                buf = torch.empty((scores.shape[0], k), dtype=torch.int32, device=scores.device)
+                buf = torch.empty((query_states.shape[0], k), dtype=torch.int32, device=query_states.device)
                 self._idx[layer_idx] = buf  # the sparse layers keep reading this very buffer
-            ops.topk(scores, k, out=buf)
+            out, _, _ = ops.dense_attn(query_states, st.k, st.v, seq_len=st.capacity, seq_lens=self._len32,
+                                       selector=selector_cls, score_len=consider_len, scale=scale, select_k=k,
+                                       idx_out=buf)
             self._sel_gen[layer_idx] = self._sel_gen.get(layer_idx, 0) + 1  # same buffer, new selection
             if self.real_offload:
                 self._stage_static(layer_idx, buf)
             return out, buf
         kview, vview = self._store[layer_idx].views()
-        out, scores = ops.dense_attn(query_states, kview, vview, selector=selector_cls, score_len=consider_len,
-                                     scale=scale)
-        idx = ops.topk(scores, min(num_selected_tokens, consider_len))
+        out, _, idx = ops.dense_attn(query_states, kview, vview, selector=selector_cls, score_len=consider_len,
+                                     scale=scale, select_k=k)
         self.set_idx_on_gpu(idx, layer_idx)
         return out, idx
 

@@ -114,7 +114,6 @@ int carve_attn_workspace(void* ws, size_t ws_bytes, int batch, int hq, int hkv, 
   return OKV_OK;
 }
 
-size_t topk_mb_workspace_bytes(int batch, int max_seq_len);
 size_t window_workspace_bytes(int batch, int hkv, int max_len);
 
 int validate_layout(const okv_kv_layout_t* layout, const void* k_base, const void* v_base) {
@@ -187,6 +186,13 @@ int okv_workspace_bytes(int op, const okv_shape_t* s, size_t* out_bytes) {
     case OKV_OP_TOPK:
       *out_bytes = okv::topk_mb_workspace_bytes(s->batch, s->max_seq_len);
       return OKV_OK;
+    case OKV_OP_DENSE_ATTN_SELECT: {  // the attention's part as the call carves it, then the selection's
+      const size_t attn = okv::attn_workspace_bytes(s->batch, s->num_q_heads, s->num_kv_heads, s->head_dim,
+                                                    s->max_seq_len, 0, s->max_seq_len, true, true, nullptr,
+                                                    nullptr);
+      *out_bytes = ((attn + 255) & ~(size_t)255) + okv::topk_mb_workspace_bytes(s->batch, s->max_seq_len);
+      return OKV_OK;
+    }
     case OKV_OP_SCORE_WINDOW:
       *out_bytes = okv::window_workspace_bytes(s->batch, s->num_kv_heads, s->max_seq_len);
       return OKV_OK;

@@ -246,24 +246,29 @@ __global__ __launch_bounds__(256) void attn_merge(RowList rows, int hq, AttnWork
 }
 
 // ------------------------------------------------------------ score finish
-// 256 threads, four consecutive tokens each, block `bx` of request `b`.  With own_lse the
+// 256 threads, TPT consecutive tokens each, block `bx` of request `b`.  With own_lse the
 // block works out the per-head score normalisers itself from the splits' partial
 // log-sum-exps (a few KB from L2) instead of reading what a merge launch left, so that it
-// does not have to run after one.
+// does not have to run after one.  Blocks of 512 tokens put twice as many CUs to pulling the
+// logits as blocks of 1024 (6.0 against 6.9 us at 128K), but each block's normalisers cost
+// Hq x splits loads, so long contexts keep the larger block.
 constexpr int kMaxFinishHeads = 256;
+template <int TPT>
 __device__ __forceinline__ void finish_body(const RowList& rows, int hq, const AttnWorkspace& w,
                                             int head_reduce, int normalise, float* __restrict__ scores,
                                             int64_t score_stride, int bx, int b, bool own_lse) {
   __shared__ float s_lse[kMaxFinishHeads];
-  const int t0 = (bx * 256 + threadIdx.x) * 4;
+  const int tid = threadIdx.x;
+  const int t0 = (bx * 256 + tid) * TPT;
   const int A = rl_score_len(rows, b);
+  if (bx * 256 * TPT >= A) return;  // the whole block: nothing below depends on the thread
   const bool is_max = head_reduce == OKV_REDUCE_MAX;
   const bool soft = normalise == OKV_NORM_SOFTMAX;
   if (soft && own_lse) {  // 8 threads per head, 32 heads per trip
     const int nA = (A + w.split_rows - 1) / w.split_rows;
-    const int sub = threadIdx.x & 7;
+    const int sub = tid & 7;
     for (int h0 = 0; h0 < hq; h0 += 32) {
-      const int h = h0 + (threadIdx.x >> 3);
+      const int h = h0 + (tid >> 3);
       float M = -INFINITY, d = 0.f;
       if (h < hq) {
         const float* pl = w.part_lse + (int64_t)(b * hq + h) * w.max_splits;
@@ -291,48 +296,59 @@ __device__ __forceinline__ void finish_body(const RowList& rows, int hq, const A
       }
       if (h < hq && sub == 0) s_lse[h] = M + log2f(d);
     }
-    __syncthreads();
   }
-  if (t0 >= A) return;
+  if (soft && own_lse) __syncthreads();
   const float init = is_max ? -INFINITY : 0.f;
-  float acc[4] = {init, init, init, init};
-  const int nh = w.logit_heads;  // Hq, or Hkv when the split pass has folded each group already
-  const float* lg = w.logits + (int64_t)b * nh * w.logits_stride + t0;
-#pragma unroll 8
-  for (int h = 0; h < nh; ++h) {
-    const float4 v4 = *reinterpret_cast<const float4*>(lg + (int64_t)h * w.logits_stride);
-    float v[4] = {v4.x, v4.y, v4.z, v4.w};
-    const float lse = soft ? (own_lse ? s_lse[h] : w.score_lse[b * hq + h]) : 0.f;
+  float acc[TPT];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      // one v_exp_f32 (a probability below 2^-126 counts as zero): with Hq exponentials per token
-      // the block's time was its arithmetic, not its loads
-      float x = soft ? __builtin_amdgcn_exp2f(fmaf(v[i], kLog2e, -lse)) : v[i];
-      acc[i] = is_max ? fmaxf(acc[i], x) : acc[i] + x;
+  for (int i = 0; i < TPT; ++i) acc[i] = init;
+  if (t0 < A) {
+    const int nh = w.logit_heads;  // Hq, or Hkv when the split pass has folded each group already
+    const float* lg = w.logits + (int64_t)b * nh * w.logits_stride + t0;
+#pragma unroll 16
+    for (int h = 0; h < nh; ++h) {
+      float v[TPT];
+      if constexpr (TPT == 4) {
+        const float4 v4 = *reinterpret_cast<const float4*>(lg + (int64_t)h * w.logits_stride);
+        v[0] = v4.x; v[1] = v4.y; v[2] = v4.z; v[3] = v4.w;
+      } else {
+        const float2 v2 = *reinterpret_cast<const float2*>(lg + (int64_t)h * w.logits_stride);
+        v[0] = v2.x; v[1] = v2.y;
+      }
+      const float lse = soft ? (own_lse ? s_lse[h] : w.score_lse[b * hq + h]) : 0.f;
+#pragma unroll
+      for (int i = 0; i < TPT; ++i) {
+        // one v_exp_f32 (a probability below 2^-126 counts as zero): with Hq exponentials per token
+        // the block's time was its arithmetic, not its loads
+        float x = soft ? __builtin_amdgcn_exp2f(fmaf(v[i], kLog2e, -lse)) : v[i];
+        acc[i] = is_max ? fmaxf(acc[i], x) : acc[i] + x;
+      }
     }
-  }
-  float* sp = scores + (int64_t)b * score_stride + t0;
-  if (t0 + 3 < A && (((uintptr_t)sp) & 15) == 0) {
-    *reinterpret_cast<float4*>(sp) = make_float4(acc[0], acc[1], acc[2], acc[3]);
-  } else {
+    float* sp = scores + (int64_t)b * score_stride + t0;
+    if (t0 + TPT - 1 < A && (((uintptr_t)sp) & (4 * TPT - 1)) == 0) {
+      if constexpr (TPT == 4) *reinterpret_cast<float4*>(sp) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+      else *reinterpret_cast<float2*>(sp) = make_float2(acc[0], acc[1]);
+    } else {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (t0 + i < A) sp[i] = acc[i];
+      for (int i = 0; i < TPT; ++i)
+        if (t0 + i < A) sp[i] = acc[i];
+    }
   }
 }
 
-// grid (ceil(max_score/1024), batch)
+// grid (ceil(max_score / (256 TPT)), batch)
+template <int TPT>
 __global__ __launch_bounds__(256) void score_finish(RowList rows, int hq, AttnWorkspace w,
                                                     int head_reduce, int normalise,
                                                     float* __restrict__ scores,
                                                     int64_t score_stride) {
-  finish_body(rows, hq, w, head_reduce, normalise, scores, score_stride, blockIdx.x, blockIdx.y, false);
+  finish_body<TPT>(rows, hq, w, head_reduce, normalise, scores, score_stride, blockIdx.x, blockIdx.y, false);
 }
 
 // Both in one launch: blocks [0, merge_blocks) fold the splits of one q head each, the rest
 // finish the scores (with their own normalisers: nothing here waits for another block).
-// grid (merge_blocks + ceil(max_score/1024), batch)
-template <typename T>
+// grid (merge_blocks + ceil(max_score / (256 TPT)), batch)
+template <typename T, int TPT>
 __global__ __launch_bounds__(256) void merge_and_finish(RowList rows, int hq, AttnWorkspace w,
                                                         T* __restrict__ out, int merge_blocks,
                                                         int head_reduce, int normalise,
@@ -341,8 +357,8 @@ __global__ __launch_bounds__(256) void merge_and_finish(RowList rows, int hq, At
   if ((int)blockIdx.x < merge_blocks)
     merge_body<T>(rows, hq, w, out, 1, 0, blockIdx.x, blockIdx.y);
   else
-    finish_body(rows, hq, w, head_reduce, normalise, scores, score_stride, blockIdx.x - merge_blocks,
-                blockIdx.y, true);
+    finish_body<TPT>(rows, hq, w, head_reduce, normalise, scores, score_stride, blockIdx.x - merge_blocks,
+                     blockIdx.y, true);
 }
 
 // ----------------------------------------------------------------- launch
@@ -401,21 +417,32 @@ static int launch_typed(const void* q, const RowList& rows, const okv_kv_layout_
     default: set_error("GQA group %d not supported", G); return OKV_ERR_UNSUPPORTED;
   }
   const bool need_score_lse = want_scores && normalise == OKV_NORM_SOFTMAX;
-  const int finish_blocks = want_scores ? (rows.max_score_len + 1023) / 1024 : 0;
+  const int ftok = finish_tokens_for(w.split_rows, rows.max_score_len);
+  const int finish_blocks = want_scores ? (rows.max_score_len + ftok - 1) / ftok : 0;
+  const AttnWorkspace& uw = *used;
   if (g_split_pass_only.load(std::memory_order_relaxed)) {
     // measurement hook: the split pass alone
   } else if (finish_blocks > 0 && hq <= kMaxFinishHeads) {
     // one launch: the merge of the outputs next to the finishing of the scores
-    hipLaunchKernelGGL((merge_and_finish<T>), dim3((with_v ? hq : 0) + finish_blocks, batch), dim3(256), 0,
-                       stream, rows, hq, *used, (T*)out, with_v ? hq : 0, head_reduce, normalise, scores,
-                       score_stride);
+    const dim3 grid((with_v ? hq : 0) + finish_blocks, batch);
+    if (ftok == 512)
+      hipLaunchKernelGGL((merge_and_finish<T, 2>), grid, dim3(256), 0, stream, rows, hq, uw, (T*)out,
+                         with_v ? hq : 0, head_reduce, normalise, scores, score_stride);
+    else
+      hipLaunchKernelGGL((merge_and_finish<T, 4>), grid, dim3(256), 0, stream, rows, hq, uw, (T*)out,
+                         with_v ? hq : 0, head_reduce, normalise, scores, score_stride);
   } else {
     if (with_v || need_score_lse)
-      hipLaunchKernelGGL((attn_merge<T>), dim3(hq, batch), dim3(256), 0, stream, rows, hq, *used,
+      hipLaunchKernelGGL((attn_merge<T>), dim3(hq, batch), dim3(256), 0, stream, rows, hq, uw,
                          (T*)out, (int)with_v, (int)need_score_lse);
-    if (finish_blocks > 0)
-      hipLaunchKernelGGL(score_finish, dim3(finish_blocks, batch), dim3(256), 0, stream, rows, hq, *used,
-                         head_reduce, normalise, scores, score_stride);
+    if (finish_blocks > 0) {
+      if (ftok == 512)
+        hipLaunchKernelGGL(score_finish<2>, dim3(finish_blocks, batch), dim3(256), 0, stream, rows, hq, uw,
+                           head_reduce, normalise, scores, score_stride);
+      else
+        hipLaunchKernelGGL(score_finish<4>, dim3(finish_blocks, batch), dim3(256), 0, stream, rows, hq, uw,
+                           head_reduce, normalise, scores, score_stride);
+    }
   }
   OKV_HIP_CHECK(hipGetLastError());
   return OKV_OK;
@@ -543,6 +570,32 @@ int okv_dense_attn(const void* q, const void* k_base, const void* v_base,
   r.max_score_len = max_score_len;
   return launch_attention(q, r, layout, batch, scale, out, true, head_reduce, normalise, scores,
                           score_stride, w, (hipStream_t)stream);
+}
+
+int okv_dense_attn_select(const void* q, const void* k_base, const void* v_base,
+                          const okv_kv_layout_t* layout, const int32_t* seq_lens, int32_t max_seq_len,
+                          int32_t batch, float scale, void* out, const int32_t* score_lens,
+                          int32_t max_score_len, int32_t head_reduce, int32_t normalise, float* scores,
+                          int64_t score_stride, const int32_t* k_per_seg, int32_t max_k,
+                          int32_t* idx_out, int64_t idx_stride, void* ws, size_t ws_bytes,
+                          okv_stream_t stream) {
+  OKV_REQUIRE(scores && idx_out, OKV_ERR_INVALID, "scores or idx_out is NULL");
+  OKV_REQUIRE(layout != nullptr, OKV_ERR_INVALID, "layout is NULL");
+  OKV_REQUIRE(batch >= 1 && max_seq_len >= 1 && max_score_len >= 0 && max_score_len <= max_seq_len,
+              OKV_ERR_INVALID, "bad batch or length");
+  // the attention's partials first, the selection's histograms and candidates behind them
+  const size_t attn_bytes = (attn_workspace_bytes(batch, layout->num_q_heads, layout->num_kv_heads,
+                                                  layout->head_dim, max_seq_len, 0, max_score_len, true, true,
+                                                  nullptr, nullptr) + 255) & ~(size_t)255;
+  OKV_REQUIRE(ws != nullptr, OKV_ERR_INVALID, "workspace pointer is NULL");
+  OKV_REQUIRE(ws_bytes >= attn_bytes, OKV_ERR_WORKSPACE, "workspace too small: have %zu, need %zu", ws_bytes,
+              attn_bytes);
+  int rc = okv_dense_attn(q, k_base, v_base, layout, seq_lens, max_seq_len, batch, scale, out, score_lens,
+                          max_score_len, head_reduce, normalise, scores, score_stride, ws, attn_bytes, stream);
+  if (rc) return rc;
+  // what is left of the workspace decides, as in okv_topk, whether long vectors get many workgroups
+  return okv_topk(scores, score_stride, score_lens, max_score_len, k_per_seg, max_k, batch, idx_out, idx_stride,
+                  (char*)ws + attn_bytes, ws_bytes - attn_bytes, stream);
 }
 
 int okv_sparse_attn(const void* q, const void* k_base, const void* v_base,

@@ -152,6 +152,16 @@ int carve_attn_workspace(void* ws, size_t ws_bytes, int batch, int hq, int hkv, 
 
 extern std::atomic<int> g_split_rows_override;  // 0 = automatic
 
+// Tokens per score-finishing block.  Every block recomputes the per-head normalisers from the
+// splits' partials, work that grows with blocks x splits: short blocks (more CUs pulling the
+// logits) while that stays small next to the logits themselves.
+inline int finish_tokens_for(int split_rows, int max_score_len) {
+  const int64_t splits = split_rows > 0 ? (max_score_len + split_rows - 1) / split_rows : 0;
+  return splits * ((max_score_len + 511) / 512) <= 65536 ? 512 : 1024;
+}
+
+size_t topk_mb_workspace_bytes(int batch, int max_seq_len);  // okv_topk_mb.hip
+
 int validate_layout(const okv_kv_layout_t* layout, const void* k_base, const void* v_base);
 
 // Implemented in okv_attn.hip.

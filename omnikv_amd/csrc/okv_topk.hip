@@ -297,7 +297,6 @@ __global__ __launch_bounds__(kThreads) void topk_select(const float* __restrict_
   }
 }
 
-size_t topk_mb_workspace_bytes(int batch, int max_seq_len);
 int launch_topk_mb(const float* scores, int64_t score_stride, const int32_t* seq_lens,
                    int32_t max_seq_len, const int32_t* k_per_seg, int32_t max_k, int32_t batch,
                    int32_t* idx_out, int64_t idx_stride, void* ws, hipStream_t stream);

@@ -24,9 +24,9 @@ HQ, HKV, D = 32, 8, 128
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--op", required=True,
-                    choices=["dense", "fused", "score", "topk", "sparse", "sparse_packed", "sparse_floor", "empty", "gather", "copy",
+                    choices=["dense", "fused", "fused_select", "fused_then_topk", "score", "topk", "sparse", "sparse_packed", "sparse_floor", "empty", "gather", "copy",
                              "offload_memcpy", "offload_zero_copy", "offload_incremental", "h2d", "window", "window_loop",
-                             "paged_dense", "paged_fused", "paged_score", "paged_topk", "paged_sparse", "paged_sparse_slots"])
+                             "paged_dense", "paged_fused", "paged_fused_select", "paged_score", "paged_topk", "paged_sparse", "paged_sparse_slots"])
     ap.add_argument("--batch", type=int, default=16, help="requests of the paged_* ops (ragged lengths 8192..32768)")
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--pages-in-order", action="store_true", help="paged_* ops: identity page table instead of shuffled")
@@ -147,6 +147,10 @@ def main():
             return ops.dense_attn(qs[l], ks[l], vs[l])
         if args.op == "fused":
             return ops.dense_attn(qs[l], ks[l], vs[l], selector=args.selector, score_len=n)
+        if args.op == "fused_select":  # the filter layer in one call
+            return ops.dense_attn(qs[l], ks[l], vs[l], selector=args.selector, score_len=n, select_k=k_sel)
+        if args.op == "fused_then_topk":  # the same as two calls
+            return ops.topk(ops.dense_attn(qs[l], ks[l], vs[l], selector=args.selector, score_len=n)[1], k_sel)
         if args.op == "score":
             return ops.score(qs[l], ks[l][:, :, :n], selector=args.selector)
         if args.op == "topk":
@@ -182,6 +186,8 @@ def main():
     algo = {
         "dense": 2.0 * (n + tail) * row,
         "fused": 2.0 * (n + tail) * row + 4.0 * n,
+        "fused_select": 2.0 * (n + tail) * row + 4.0 * n + 4.0 * k_sel,
+        "fused_then_topk": 2.0 * (n + tail) * row + 4.0 * n + 4.0 * k_sel,
         "score": 1.0 * n * row + 4.0 * n,
         "topk": 4.0 * n + 4.0 * k_sel,
         "window": 1.0 * n * row + 4.0 * n,  # one reading of K; the kernels read it twice
@@ -270,6 +276,9 @@ def paged(args, dev):
         if args.op == "paged_fused":
             return dense_(qs[l], pools[l], seq_len=nmax, seq_lens=lens_d, selector=args.selector,
                                   score_len=nmax, score_lens=lens_d)
+        if args.op == "paged_fused_select":
+            return dense_(qs[l], pools[l], seq_len=nmax, seq_lens=lens_d, selector=args.selector, score_len=nmax,
+                          score_lens=lens_d, select_k=kmax, k_per_seg=k_per_d)
         if args.op == "paged_score":
             return score_(qs[l], pools[l], score_len=nmax, selector=args.selector, score_lens=lens_d)
         if args.op == "paged_topk":
@@ -281,6 +290,7 @@ def paged(args, dev):
     tokens, sel = int(lens.sum()), int(k_per.sum())
     row = HKV * D * es
     algo = {"paged_dense": 2.0 * tokens * row, "paged_fused": 2.0 * tokens * row + 4.0 * tokens,
+            "paged_fused_select": 2.0 * tokens * row + 4.0 * tokens + 4.0 * sel,
             "paged_score": 1.0 * tokens * row + 4.0 * tokens, "paged_topk": 4.0 * tokens + 4.0 * sel,
             "paged_sparse": 2.0 * sel * row + 4.0 * sel, "paged_sparse_slots": 2.0 * sel * row + 4.0 * sel}[args.op]
     for i in range(args.warmup):

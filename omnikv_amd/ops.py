@@ -229,9 +229,13 @@ def topk(scores: torch.Tensor, k: int, seq_lens: Optional[torch.Tensor] = None,
 def dense_attn(q, k, v=None, seq_len: Optional[int] = None, seq_lens: Optional[torch.Tensor] = None,
                scale: Optional[float] = None, selector: Optional[str] = None,
                score_len: Optional[int] = None, score_lens: Optional[torch.Tensor] = None,
-               scores_out: Optional[torch.Tensor] = None):
+               scores_out: Optional[torch.Tensor] = None, select_k: Optional[int] = None,
+               k_per_seg: Optional[torch.Tensor] = None, idx_out: Optional[torch.Tensor] = None):
     """Dense GQA decode attention; with `selector` also returns the filter-layer
-    scores of the first score_len tokens from the same pass.  okv_dense_attn."""
+    scores of the first score_len tokens from the same pass (okv_dense_attn), and with
+    `select_k` on top of that the ascending indices of the select_k largest of them, as
+    topk(scores, select_k, score_lens, k_per_seg) would: (out, scores, idx), the whole filter
+    layer in one call (okv_dense_attn_select)."""
     q = _q3(q)
     _require_gpu(q, "q")
     hq, d = q.shape[1], q.shape[2]
@@ -244,6 +248,8 @@ def dense_attn(q, k, v=None, seq_len: Optional[int] = None, seq_lens: Optional[t
     out = torch.empty_like(q)
     scores = None
     sp, ss, red, norm = None, 0, 0, 0
+    if select_k is not None and selector is None:
+        raise ValueError("select_k needs a selector")
     if selector is not None:
         norm_s, red_s = SELECTOR_MODES[selector]
         red, norm = _REDUCE[red_s], _NORM[norm_s]
@@ -255,15 +261,34 @@ def dense_attn(q, k, v=None, seq_len: Optional[int] = None, seq_lens: Optional[t
         elif scores.shape != (batch, score_len) or scores.dtype != torch.float32 or scores.stride(1) != 1:
             raise ValueError("scores_out must be (bsz, score_len) float32 with contiguous rows")
         sp, ss = scores.data_ptr(), scores.stride(0)
-    nbytes = workspace_bytes(_lib.OKV_OP_DENSE_ATTN, batch, hq, lay.num_kv_heads, d, seq_len,
-                             with_scores=selector is not None)
+    sc = scale if scale is not None else 1.0 / math.sqrt(d)
+    if select_k is None:
+        nbytes = workspace_bytes(_lib.OKV_OP_DENSE_ATTN, batch, hq, lay.num_kv_heads, d, seq_len,
+                                 with_scores=selector is not None)
+        ws = _workspace(q.device, nbytes)
+        check(lib().okv_dense_attn(
+            q.data_ptr(), kp, vp, C.byref(lay), _lens(seq_lens, batch, "seq_lens"), seq_len, batch,
+            sc, out.data_ptr(), _lens(score_lens, batch, "score_lens"), score_len or 0, red, norm, sp, ss,
+            ws.data_ptr(), ws.numel(), _stream_ptr(q.device)))
+        return (out, scores) if selector is not None else out
+    kk = min(select_k, score_len)
+    idx = idx_out
+    if idx is None:
+        if score_lens is None and k_per_seg is None:
+            idx = torch.empty((batch, kk), dtype=torch.int32, device=q.device)
+        else:  # ragged: entries beyond a request's own k are left untouched -> padding is -1
+            idx = torch.full((batch, kk), -1, dtype=torch.int32, device=q.device)
+    elif idx.shape != (batch, kk) or idx.dtype != torch.int32 or idx.stride(1) != 1:
+        raise ValueError("idx_out must be (bsz, min(select_k, score_len)) int32 with contiguous rows")
+    nbytes = workspace_bytes(_lib.OKV_OP_DENSE_ATTN_SELECT, batch, hq, lay.num_kv_heads, d, seq_len,
+                             with_scores=True)
     ws = _workspace(q.device, nbytes)
-    check(lib().okv_dense_attn(
+    check(lib().okv_dense_attn_select(
         q.data_ptr(), kp, vp, C.byref(lay), _lens(seq_lens, batch, "seq_lens"), seq_len, batch,
-        scale if scale is not None else 1.0 / math.sqrt(d), out.data_ptr(),
-        _lens(score_lens, batch, "score_lens"), score_len or 0, red, norm, sp, ss,
+        sc, out.data_ptr(), _lens(score_lens, batch, "score_lens"), score_len, red, norm, sp, ss,
+        _lens(k_per_seg, batch, "k_per_seg"), select_k, idx.data_ptr(), idx.stride(0),
         ws.data_ptr(), ws.numel(), _stream_ptr(q.device)))
-    return (out, scores) if selector is not None else out
+    return out, scores, idx
 
 
 def sparse_attn(q, k, v=None, idx: Optional[torch.Tensor] = None, sel_len: Optional[int] = None,

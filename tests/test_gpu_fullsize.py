@@ -61,6 +61,9 @@ def test_filter_layer_op_matches_oracle_at_benchmark_size(n, ks):
             # identical fp32 scores -> identical indices
             idx = ops.topk(want.to(DEV), kk)
             assert torch.equal(idx.cpu().to(torch.int64), want_idx), (sel, kk)
+            # attention, scores and selection in one call: the same bits as the separate calls
+            out1, sc1, idx1 = ops.dense_attn(qd, kd, vd, selector=sel, score_len=n, select_k=kk)
+            assert torch.equal(out1, out) and torch.equal(sc1, fused) and torch.equal(idx1, ops.topk(fused, kk))
             # the kernels' own scores: differences are near-ties only
             for got in (alone, fused):
                 own = ops.topk(got, kk).cpu()[0].to(torch.int64)
@@ -121,6 +124,9 @@ def test_batch16_ragged_paged_matches_oracle_at_benchmark_size():
         # ragged top-k on the ORACLE's scores: bit-exact, padding -1
         idx = ops.topk(want_scores.to(DEV), kmax, seq_lens=lens_d, k_per_seg=k_per.to(DEV))
         own = ops.topk(fused, kmax, seq_lens=lens_d, k_per_seg=k_per.to(DEV)).cpu()
+        out1, sc1, idx1 = ops.dense_attn(q, kv, seq_len=nmax, seq_lens=lens_d, selector=sel, score_len=nmax,
+                                         score_lens=lens_d, select_k=kmax, k_per_seg=k_per.to(DEV))
+        assert torch.equal(out1, out) and torch.equal(idx1.cpu(), own)  # the one-call filter layer
         slots = kv.slot_index(idx)
         sparse = ops.sparse_attn(qn.to(DEV), kv, idx=idx, sel_len=kmax, sel_lens=k_per.to(DEV))
         via_slots = ops.sparse_attn(qn.to(DEV), kv, slots=slots, sel_len=kmax, sel_lens=k_per.to(DEV))

@@ -160,6 +160,62 @@ def test_dense_attention_with_fused_scores(selector, dtype):
     assert _rel_err(scores.cpu(), alone.cpu()) < 1e-5
 
 
+@pytest.mark.parametrize("selector", ["last", "softmax_sum_last"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,consider,ksel", [(4096 + 37, 4096, 274), (14336, 14336, 960), (20011, 20000, 1340),
+                                              (70001, 69990, 4689), (70001, 69990, 69990), (40000, 39999, 1)])
+def test_filter_layer_in_one_call_equals_attention_then_topk(selector, dtype, n, consider, ksel):
+    """okv_dense_attn_select against okv_dense_attn followed by okv_topk on the same inputs: the same
+    bits in all three outputs (below and above the length at which top-k goes to many workgroups),
+    and the indices against the oracle's stable top-k of those scores."""
+    q, k, v, kd, vd = _inputs(n, dtype, "hf")
+    qd = q.to(DEV)
+    out2, scores2 = ops.dense_attn(qd, kd, vd, selector=selector, score_len=consider)
+    idx2 = ops.topk(scores2, ksel)
+    for _ in range(2):  # the second call finds the workspace as the first left it
+        out1, scores1, idx1 = ops.dense_attn(qd, kd, vd, selector=selector, score_len=consider, select_k=ksel)
+        assert torch.equal(out1, out2) and torch.equal(scores1, scores2)
+        assert torch.equal(idx1, idx2)
+    want = orc.select_topk_stable(scores1.cpu(), ksel)
+    assert torch.equal(idx1.cpu().to(torch.int64), want)
+
+
+def test_filter_layer_in_one_call_ragged_batch_and_both_block_sizes():
+    """Requests of different lengths (one empty, one shorter than a score-finishing block, two ending
+    inside one) with per-request k, at the automatic split size and at one small enough that the
+    score-finishing blocks take 1024 tokens instead of 512."""
+    from omnikv_amd._lib import check, lib
+    g = torch.Generator().manual_seed(77)
+    lens = torch.tensor([30000, 0, 300, 16385, 24577], dtype=torch.int32)
+    ks = torch.tensor([2010, 5, 20, 16385, 0], dtype=torch.int32)
+    hq, hkv, d, nmax = 32, 8, 128, int(lens.max())
+    k = torch.randn((len(lens), hkv, nmax + 1, d), generator=g).to(torch.bfloat16)
+    v = torch.randn((len(lens), hkv, nmax + 1, d), generator=g).to(torch.bfloat16)
+    q = torch.randn((len(lens), hq, 1, d), generator=g).to(torch.bfloat16)
+    kd, vd, qd, ld, ksd = k.to(DEV), v.to(DEV), q.to(DEV), lens.to(DEV), ks.to(DEV)
+    seq = (lens + 1).to(DEV)  # every request attends to one row more than is scored
+    kmax = int(ks.max())
+    try:
+        for split_rows in (0, 64):
+            check(lib().okv_set_option(b"split_rows", split_rows))
+            for sel in ("last", "softmax_sum_last"):
+                out2, sc2 = ops.dense_attn(qd, kd, vd, seq_len=nmax + 1, seq_lens=seq, selector=sel, score_len=nmax,
+                                           score_lens=ld)
+                idx2 = ops.topk(sc2, kmax, seq_lens=ld, k_per_seg=ksd)
+                out1, sc1, idx1 = ops.dense_attn(qd, kd, vd, seq_len=nmax + 1, seq_lens=seq, selector=sel,
+                                                 score_len=nmax, score_lens=ld, select_k=kmax, k_per_seg=ksd)
+                assert torch.equal(out1, out2)
+                for b, n in enumerate(int(x) for x in lens):
+                    kb = min(int(ks[b]), n)
+                    assert torch.equal(sc1[b, :n], sc2[b, :n])
+                    assert torch.equal(idx1[b, :kb], idx2[b, :kb]), (split_rows, sel, b)
+                    assert (idx1[b, kb:] == -1).all()
+                    want = orc.select_topk_stable(sc1[b:b + 1, :n].cpu(), kb)[0]
+                    assert torch.equal(idx1[b, :kb].cpu().to(torch.int64), want), (split_rows, sel, b)
+    finally:
+        check(lib().okv_set_option(b"split_rows", 0))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("layout", ["hf", "token_major"])
 @pytest.mark.parametrize("n,ksel,tail", [(4096, 274, 0), (4096, 274, 5), (4096, 1, 1), (20000, 1340, 100),
