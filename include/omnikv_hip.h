@@ -66,7 +66,8 @@ enum okv_op {
   OKV_OP_DENSE_ATTN = 2, /* with or without the fused score output */
   OKV_OP_SPARSE_ATTN = 3,
   OKV_OP_SCORE_WINDOW = 4,
-  OKV_OP_DENSE_ATTN_SELECT = 5
+  OKV_OP_DENSE_ATTN_SELECT = 5,
+  OKV_OP_DENSE_ATTN_WINDOW = 6
 };
 
 typedef struct okv_kv_layout {
@@ -150,6 +151,27 @@ int okv_score_window(const void* q, int64_t q_batch_stride, int64_t q_head_strid
                      const okv_kv_layout_t* layout, const int32_t* score_lens,
                      int32_t max_score_len, int32_t batch, float scale, float* scores,
                      int64_t score_stride, void* ws, size_t ws_bytes, okv_stream_t stream);
+
+/*
+ * A filter layer with a window selector in two passes over K instead of three: the dense
+ * attention of okv_dense_attn (q: the current position's query, (batch, num_q_heads, head_dim))
+ * and the window scores of okv_score_window (q_window, window, exp_decay: as there; its last
+ * position is the current one) over the first score_len tokens.  The attention's pass over K
+ * and V also computes every window column's log-sum-exp, which is the first of
+ * okv_score_window's two passes; the second follows.  out and scores as from the two calls
+ * (scores to rounding: the partial sums are grouped by the attention's splits).
+ * score_lens[b] must not exceed seq_lens[b].  Same restrictions as okv_score_window.
+ * Replaces, for the selectors `uniform` and `exp`, select_tokens_by_attn_universal
+ * (modeling/omnikv.py:59-103, called at :189-198) and the attention of the same layer at
+ * :219-227.  Workspace: okv_workspace_bytes(OKV_OP_DENSE_ATTN_WINDOW, ...).
+ */
+int okv_dense_attn_window(const void* q, const void* q_window, int64_t q_batch_stride,
+                          int64_t q_head_stride, int64_t q_pos_stride, int32_t window,
+                          int32_t exp_decay, const void* k_base, const void* v_base,
+                          const okv_kv_layout_t* layout, const int32_t* seq_lens,
+                          int32_t max_seq_len, int32_t batch, float scale, void* out,
+                          const int32_t* score_lens, int32_t max_score_len, float* scores,
+                          int64_t score_stride, void* ws, size_t ws_bytes, okv_stream_t stream);
 
 /*
  * Per-request top-k of fp32 scores.  Writes the k_b = min(k_per_seg[b], len_b)

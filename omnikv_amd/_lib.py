@@ -16,7 +16,7 @@ OKV_F32, OKV_BF16, OKV_F16 = 0, 1, 2
 OKV_REDUCE_MAX, OKV_REDUCE_SUM = 0, 1
 OKV_NORM_RAW, OKV_NORM_SOFTMAX = 0, 1
 OKV_OP_SCORE, OKV_OP_TOPK, OKV_OP_DENSE_ATTN, OKV_OP_SPARSE_ATTN, OKV_OP_SCORE_WINDOW = 0, 1, 2, 3, 4
-OKV_OP_DENSE_ATTN_SELECT = 5
+OKV_OP_DENSE_ATTN_SELECT, OKV_OP_DENSE_ATTN_WINDOW = 5, 6
 
 EXPORTS = (
     "okv_strerror",
@@ -29,6 +29,7 @@ EXPORTS = (
     "okv_topk",
     "okv_dense_attn",
     "okv_dense_attn_select",
+    "okv_dense_attn_window",
     "okv_sparse_attn",
     "okv_sparse_attn_noalloc",
     "okv_noalloc_scratch_bytes",
@@ -109,6 +110,9 @@ def _declare(l):
     l.okv_dense_attn.argtypes = [vp, vp, vp, C.POINTER(KVLayout), vp, i32, i32, f32, vp, vp, i32, i32, i32, vp, i64, vp, sz, vp]
     l.okv_dense_attn_select.restype = C.c_int
     l.okv_dense_attn_select.argtypes = l.okv_dense_attn.argtypes[:-3] + [vp, i32, vp, i64, vp, sz, vp]
+    l.okv_dense_attn_window.restype = C.c_int
+    l.okv_dense_attn_window.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, vp, C.POINTER(KVLayout), vp, i32, i32, f32,
+                                        vp, vp, i32, vp, i64, vp, sz, vp]
     l.okv_sparse_attn.restype = C.c_int
     l.okv_sparse_attn.argtypes = [vp, vp, vp, C.POINTER(KVLayout), vp, i64, vp, i32, vp, vp, i64, i64, i64, vp, i32, i32, f32, vp, vp, sz, vp]
     l.okv_sparse_attn_noalloc.restype = C.c_int

@@ -622,6 +622,46 @@ class OmniKVMultiStageCache:
             self._stage_static(layer_idx, buf)
         return buf
 
+    def attend_and_select_window(self, query_states: torch.Tensor, query_window: torch.Tensor, layer_idx: int,
+                                 num_selected_tokens: int, consider_len: int, selector_cls: str, forced_tail: int = 0,
+                                 scale: Optional[float] = None):
+        """Filter layer with a window selector (`uniform` / `exp`) whose first scoring pass rides on the
+        layer's own attention: what select_with_query followed by attend do, in two passes over K
+        instead of three.  query_states: (bsz, Hq, 1, D), the attention's query; query_window:
+        (bsz, Hq, W, D), rotated.  Returns (attention output, idx int32 (bsz, k)).  Operands the
+        kernel does not take (fp32, more than 64 window columns per kv head) go the separate way."""
+        st = self._store[layer_idx]
+        if not ops.window_supported(query_window, st.k):
+            idx = self.select_with_query(query_window, layer_idx, num_selected_tokens, consider_len, selector_cls,
+                                         forced_tail=forced_tail)
+            return self.attend(query_states, layer_idx, scale=scale), idx
+        k = min(num_selected_tokens, consider_len)
+        if self._static:
+            if forced_tail:
+                raise RuntimeError("static decode with a window selector starts once the window has left the prompt")
+            out, scores = ops.dense_attn_window(query_states, query_window, st.k, st.v, selector=selector_cls,
+                                                seq_len=st.capacity, seq_lens=self._len32, score_len=consider_len,
+                                                scale=scale)
+            buf = self._idx.get(layer_idx)
+            if buf is None or buf.shape[1] != k:
+                buf = torch.empty((scores.shape[0], k), dtype=torch.int32, device=scores.device)
+                self._idx[layer_idx] = buf  # the sparse layers keep reading this very buffer
+            ops.topk(scores, k, out=buf)
+            self._sel_gen[layer_idx] = self._sel_gen.get(layer_idx, 0) + 1
+            if self.real_offload:
+                self._stage_static(layer_idx, buf)
+            return out, buf
+        kview, vview = st.views()
+        out, scores = ops.dense_attn_window(query_states, query_window, kview, vview, selector=selector_cls,
+                                            score_len=consider_len, scale=scale)
+        idx = ops.topk(scores, k).to(torch.int64)
+        if forced_tail:
+            end = consider_len + forced_tail
+            tail_idx = torch.arange(end - forced_tail, end, device=idx.device)
+            idx = torch.cat([idx, tail_idx[None, :].repeat(idx.shape[0], 1)], dim=1)
+        self.set_idx_on_gpu(idx, layer_idx)
+        return out, self._idx[layer_idx]
+
     def attend_and_select(self, query_states: torch.Tensor, layer_idx: int, num_selected_tokens: int,
                           consider_len: int, selector_cls: str = "last", scale: Optional[float] = None):
         """Filter layer: dense attention, the filter-layer scores from the same pass over K and

@@ -41,17 +41,18 @@ static int num_compute_units() {
 // scoring alone could hold five and does best sized for three (measured at 128K: 50.6 us against
 // 53.1 sized for six).  The cap keeps the LDS staging of a scored split's logits small.
 static int choose_split_rows(int batch, int hq, int hkv, int total_rows, bool with_v,
-                             bool with_logits, bool gather) {
+                             bool with_logits, int kind) {
   const int forced = g_split_rows_override.load(std::memory_order_relaxed);
   if (forced > 0) return forced;
-  (void)gather;
   // a batch is sized by its longest request, so ragged ones fill less than the grid suggests:
   // three and six per CU there (measured on 16 requests of 8K..32K tokens)
-  const int64_t capacity = (int64_t)num_compute_units() * (batch <= 1 ? (with_v ? 2 : 3) : (with_v ? 3 : 6));
+  // kind 2: the dense pass that carries a query window needs more than half a SIMD's registers per wave, so
+  // one workgroup per CU is resident
+  const int64_t capacity = (int64_t)num_compute_units() * (kind == 2 ? 1 : batch <= 1 ? (with_v ? 2 : 3) : (with_v ? 3 : 6));
   // a scored split stages G*rows fp32 logits in LDS: keep that within 33 KB (2112 rows at G = 4,
   // what one round of a 128K context needs)
   const int group = hkv > 0 && hq >= hkv ? hq / hkv : 1;
-  const int64_t cap_rows = with_logits ? (8448 / group) / 64 * 64 : 4096;
+  const int64_t cap_rows = with_logits ? (8448 / group) / 64 * 64 : kind == 2 ? 8192 : 4096;
   const int64_t work = (int64_t)(total_rows > 0 ? total_rows : 1) * hkv * (batch > 0 ? batch : 1);
   for (int64_t rounds = 1;; ++rounds) {
     int64_t rows = (work + rounds * capacity - 1) / (rounds * capacity);
@@ -67,9 +68,9 @@ static int choose_split_rows(int batch, int hq, int hkv, int total_rows, bool wi
 
 size_t attn_workspace_bytes(int batch, int hq, int hkv, int d, int max_main, int max_tail,
                             int max_score, bool with_v, bool with_logits, int* split_rows,
-                            int* max_splits, bool gather) {
+                            int* max_splits, int kind) {
   int L = max_main + max_tail;
-  int C = choose_split_rows(batch, hq, hkv, L, with_v, with_logits, gather);
+  int C = choose_split_rows(batch, hq, hkv, L, with_v, with_logits, kind);
   int S = (L + C - 1) / C + (max_score > 0 ? 1 : 0);
   if (S < 1) S = 1;
   if (split_rows) *split_rows = C;
@@ -87,10 +88,10 @@ size_t attn_workspace_bytes(int batch, int hq, int hkv, int d, int max_main, int
 
 int carve_attn_workspace(void* ws, size_t ws_bytes, int batch, int hq, int hkv, int d,
                          int max_main, int max_tail, int max_score, bool with_v,
-                         bool with_logits, AttnWorkspace* out, bool gather) {
+                         bool with_logits, AttnWorkspace* out, int kind) {
   int C = 0, S = 0;
   size_t need = attn_workspace_bytes(batch, hq, hkv, d, max_main, max_tail, max_score, with_v,
-                                     with_logits, &C, &S, gather);
+                                     with_logits, &C, &S, kind);
   OKV_REQUIRE(ws != nullptr, OKV_ERR_INVALID, "workspace pointer is NULL");
   OKV_REQUIRE(ws_bytes >= need, OKV_ERR_WORKSPACE, "workspace too small: have %zu, need %zu",
               ws_bytes, need);
@@ -115,6 +116,7 @@ int carve_attn_workspace(void* ws, size_t ws_bytes, int batch, int hq, int hkv, 
 }
 
 size_t window_workspace_bytes(int batch, int hkv, int max_len);
+size_t dense_window_workspace_bytes(int batch, int hq, int hkv, int d, int max_seq_len, int max_score_len);
 
 int validate_layout(const okv_kv_layout_t* layout, const void* k_base, const void* v_base) {
   OKV_REQUIRE(layout != nullptr, OKV_ERR_INVALID, "layout is NULL");
@@ -193,6 +195,10 @@ int okv_workspace_bytes(int op, const okv_shape_t* s, size_t* out_bytes) {
       *out_bytes = ((attn + 255) & ~(size_t)255) + okv::topk_mb_workspace_bytes(s->batch, s->max_seq_len);
       return OKV_OK;
     }
+    case OKV_OP_DENSE_ATTN_WINDOW:
+      *out_bytes = okv::dense_window_workspace_bytes(s->batch, s->num_q_heads, s->num_kv_heads, s->head_dim,
+                                                     s->max_seq_len, s->max_seq_len);
+      return OKV_OK;
     case OKV_OP_SCORE_WINDOW:
       *out_bytes = okv::window_workspace_bytes(s->batch, s->num_kv_heads, s->max_seq_len);
       return OKV_OK;

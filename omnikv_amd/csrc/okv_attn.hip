@@ -467,7 +467,27 @@ int launch_attention(const void* q, const RowList& rows, const okv_kv_layout_t* 
   return OKV_ERR_UNSUPPORTED;
 }
 
-static void fill_main(RowList* r, const void* k, const void* v, const okv_kv_layout_t* lay) {
+bool launch_stage1_window(int dtype, const void* q, const RowList& rows, int hq, int hkv, int batch, float scale,
+                          const AttnWorkspace& w, const WindowFuse& wf, hipStream_t stream);
+
+// Dense attention of 16-bit contiguous K/V whose split pass also leaves the window columns'
+// partial log-sum-exps (see WindowFuse); the merge of the attention output follows.
+int launch_attention_window(const void* q, const RowList& rows, const okv_kv_layout_t* lay, int batch, float scale,
+                            void* out, const AttnWorkspace& w, const WindowFuse& wf, hipStream_t stream) {
+  const int hq = lay->num_q_heads, hkv = lay->num_kv_heads;
+  if (!launch_stage1_window(lay->dtype, q, rows, hq, hkv, batch, scale, w, wf, stream)) {
+    set_error("window scoring inside the dense pass needs 16-bit contiguous K/V and window x group <= %d", kWinCols);
+    return OKV_ERR_UNSUPPORTED;
+  }
+  if (lay->dtype == OKV_BF16)
+    hipLaunchKernelGGL((attn_merge<BF16>), dim3(hq, batch), dim3(256), 0, stream, rows, hq, w, (BF16*)out, 1, 0);
+  else
+    hipLaunchKernelGGL((attn_merge<F16>), dim3(hq, batch), dim3(256), 0, stream, rows, hq, w, (F16*)out, 1, 0);
+  OKV_HIP_CHECK(hipGetLastError());
+  return OKV_OK;
+}
+
+void fill_main(RowList* r, const void* k, const void* v, const okv_kv_layout_t* lay) {
   memset(r, 0, sizeof(*r));
   r->k_base = k;
   r->v_base = v;

@@ -82,6 +82,7 @@ template <int G>
 __host__ __device__ constexpr int stage1_lds_floats(bool with_v) {
   return 3 * 16 * G + 16 + (with_v ? 16 * G * kD : 0);
 }
+constexpr int kWindowLdsFloats = 2 * 16 * kWinCols;  // [16 lane rows][64 columns] running max and sum
 
 // The streaming modes (0, 3) load K as whole rows and transpose the tile in LDS (see
 // k_rows_to_a_operand); the gather modes keep the direct A-operand loads: their pass is a
@@ -91,9 +92,12 @@ __host__ __device__ constexpr bool stage1_k_through_lds(int mode) { return mode 
 // MODE 0: contiguous rows, no index, no tail.  MODE 1: rows through idx (no page table),
 // optional tail.  MODE 2: anything (page tables, idx or not, tail or not).  MODE 3: page
 // table with pages of 2^n >= 16 rows, no index, no tail (a tile never straddles a page).
-template <typename T, int G, bool WITH_V, int MODE, bool LOGITS>
-__global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q, RowList rows,
-                                                        int hq, float scale, AttnWorkspace w) {
+// WINDOW: the tiles of the scored splits also meet the W x G window query rows of the kv head
+// (four more 16-column B operands: column c is position c / G, q head g*G + c % G) and every
+// column keeps the running max and sum of its logits; nothing else changes.
+template <typename T, int G, bool WITH_V, int MODE, bool LOGITS, bool WINDOW>
+__device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const RowList& rows, int hq, float scale,
+                                                 const AttnWorkspace& w, const WindowFuse& wf) {
   extern __shared__ float lds[];
   constexpr bool KLDS = stage1_k_through_lds(MODE);
   const int g = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
@@ -116,6 +120,28 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
     for (int s = 0; s < 4; ++s) {
       const uint4 v = *reinterpret_cast<const uint4*>(qp + 32 * s);
       qf[s] = r16 < G ? v : make_uint4(0, 0, 0, 0);
+    }
+  }
+
+  constexpr int WCB = WINDOW ? kWinCols / 16 : 1;
+  uint4 wqf[WCB][4];
+  float wm[WCB], wl[WCB];  // per column block: state of (column r16, lane row j4), max in raw units
+  const bool wscored = WINDOW && begin < A;  // a scored split ends at or before A
+  if (WINDOW) {
+#pragma unroll
+    for (int cb = 0; cb < WCB; ++cb) {
+      const int c = 16 * cb + r16;
+      const int wpos = c / G, hg = c % G;
+      const bool valid = wpos < wf.window;
+      const T* qp = reinterpret_cast<const T*>(wf.wq) + (int64_t)b * wf.q_batch_stride +
+                    (int64_t)(g * G + hg) * wf.q_head_stride + (int64_t)(valid ? wpos : 0) * wf.q_pos_stride + 8 * j4;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const uint4 v = *reinterpret_cast<const uint4*>(qp + 32 * s);
+        wqf[cb][s] = valid ? v : make_uint4(0, 0, 0, 0);
+      }
+      wm[cb] = -INFINITY;
+      wl[cb] = 0.f;
     }
   }
 
@@ -219,6 +245,8 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
   // K staging of the streaming modes: 4 KB per wave behind everything else the block keeps in LDS
   int kst_off = stage1_lds_floats<G>(WITH_V);
   if (LOGITS && G * w.split_rows > kst_off) kst_off = G * w.split_rows;
+  float* wlds = lds + kst_off;  // the window columns' states meet here at the end
+  if (WINDOW) kst_off += kWindowLdsFloats;
   char* kstage = reinterpret_cast<char*>(lds + kst_off) + wave * 4096;
   auto compute = [&](int tbase, const uint4 (&kf_in)[4], const uint4 (&vf)[4]) {
     uint4 kf[4];
@@ -233,6 +261,31 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
     for (int s = 0; s < 4; ++s) S = mfma16((const T*)nullptr, kf[s], qf[s], S);
     const int row0 = tbase + 4 * j4;
     const bool partial = tbase + 16 > end;  // wave-uniform
+    if (WINDOW) {
+      if (wscored) {
+#pragma unroll
+        for (int cb = 0; cb < WCB; ++cb) {
+          f32x4_t W = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int s = 0; s < 4; ++s) W = mfma16((const T*)nullptr, kf[s], wqf[cb][s], W);
+          float sv[4] = {W[0], W[1], W[2], W[3]};
+          if (partial) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (row0 + i >= end) sv[i] = -INFINITY;
+          }
+          const float mn = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), wm[cb]);
+          const float ms = mn == -INFINITY ? 0.f : mn;
+          const float neg = -ms * sl2;
+          const float alpha = __builtin_amdgcn_exp2f((wm[cb] - ms) * sl2);
+          float pw = 0.f;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) pw += __builtin_amdgcn_exp2f(fmaf(sv[i], sl2, neg));
+          wl[cb] = fmaf(wl[cb], alpha, pw);
+          wm[cb] = mn;
+        }
+      }
+    }
     if (scored) {  // staged in LDS, flushed after the loop: no global store in the loop
       float v[4] = {S[0] * scale, S[1] * scale, S[2] * scale, S[3] * scale};
       if (w.group_reduce) {  // raw scores: fold the G q heads (lanes 0..G-1 of the lane row) here
@@ -386,7 +439,33 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
       dst[1] = make_float4(acc[h][4], acc[h][5], acc[h][6], acc[h][7]);
     }
   }
+  if (WINDOW) {
+    if (wscored) {
+#pragma unroll
+      for (int cb = 0; cb < WCB; ++cb) {
+        wlds[grp * kWinCols + 16 * cb + r16] = wm[cb];
+        wlds[16 * kWinCols + grp * kWinCols + 16 * cb + r16] = wl[cb];
+      }
+    }
+  }
   __syncthreads();
+  if (WINDOW) {
+    if (wscored && threadIdx.x < kWinCols) {
+      const int c = threadIdx.x;
+      float M = -INFINITY;
+#pragma unroll
+      for (int x = 0; x < 16; ++x) M = fmaxf(M, wlds[x * kWinCols + c]);
+      float den = 0.f;
+#pragma unroll
+      for (int x = 0; x < 16; ++x) {
+        const float mm = wlds[x * kWinCols + c];
+        den = fmaf(wlds[16 * kWinCols + x * kWinCols + c], mm == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((mm - M) * sl2),
+                   den);
+      }
+      wf.part[((int64_t)(b * (hq / G) + g) * kWinCols + c) * w.max_splits + split] =
+          M == -INFINITY ? -INFINITY : M * sl2 + log2f(den);
+    }
+  }
   for (int o = threadIdx.x; o < G * kD; o += 256) {
     const int h = o / kD, d = o % kD;
     float M = -INFINITY;
@@ -407,23 +486,45 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
 }
 
 template <typename T, int G, bool WITH_V, int MODE, bool LOGITS>
+__global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q, RowList rows,
+                                                        int hq, float scale, AttnWorkspace w) {
+  stage1_mfma_body<T, G, WITH_V, MODE, LOGITS, false>(q, rows, hq, scale, w, WindowFuse{});
+}
+
+// The dense pass with the window columns: capped at the registers that let two workgroups share a
+// CU, like the pass without them.
+template <typename T, int G>
+__global__ __launch_bounds__(256) void attn_stage1_window_mfma(const T* __restrict__ q, RowList rows,
+                                                                  int hq, float scale, AttnWorkspace w,
+                                                                  WindowFuse wf) {
+  stage1_mfma_body<T, G, true, 0, false, true>(q, rows, hq, scale, w, wf);
+}
+
+template <typename T, int G, bool WITH_V, int MODE, bool LOGITS, bool WINDOW = false>
 static void launch_one(const void* q, const RowList& rows, int hq, int hkv, int batch, float scale,
-                       const AttnWorkspace& w, hipStream_t stream) {
-  auto kern = attn_stage1_mfma<T, G, WITH_V, MODE, LOGITS>;
+                       const AttnWorkspace& w, hipStream_t stream, const WindowFuse& wf = WindowFuse{}) {
+  const void* kern_ptr;
+  if constexpr (WINDOW) kern_ptr = reinterpret_cast<const void*>(attn_stage1_window_mfma<T, G>);
+  else kern_ptr = reinterpret_cast<const void*>(attn_stage1_mfma<T, G, WITH_V, MODE, LOGITS>);
   size_t lds_floats = stage1_lds_floats<G>(WITH_V);  // the logits staging aliases the merge buffers
   if (LOGITS && (size_t)G * w.split_rows > lds_floats) lds_floats = (size_t)G * w.split_rows;
+  if (WINDOW) lds_floats += kWindowLdsFloats;
   if (stage1_k_through_lds(MODE)) lds_floats += 4 * 1024;  // 4 KB of K staging per wave
   const size_t lds_bytes = lds_floats * sizeof(float);
   static std::atomic<size_t> configured{0};  // per instantiation; two threads raising it at once both succeed
   if (lds_bytes > configured.load(std::memory_order_relaxed)) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    (void)hipFuncSetAttribute(kern_ptr, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     size_t seen = configured.load(std::memory_order_relaxed);
     while (seen < lds_bytes && !configured.compare_exchange_weak(seen, lds_bytes, std::memory_order_relaxed)) {
     }
   }
   dim3 grid(hkv, w.max_splits, batch);  // kv head fastest: co-resident blocks cover whole token rows
-  hipLaunchKernelGGL(kern, grid, dim3(256), lds_bytes, stream, (const T*)q, rows, hq, scale, w);
+  if constexpr (WINDOW)
+    hipLaunchKernelGGL((attn_stage1_window_mfma<T, G>), grid, dim3(256), lds_bytes, stream, (const T*)q, rows, hq,
+                       scale, w, wf);
+  else
+    hipLaunchKernelGGL((attn_stage1_mfma<T, G, WITH_V, MODE, LOGITS>), grid, dim3(256), lds_bytes, stream,
+                       (const T*)q, rows, hq, scale, w);
 }
 
 template <typename T, int G>
@@ -626,6 +727,33 @@ bool launch_score_raw_mfma(int dtype, const void* q, const RowList& rows, int hq
     return launch_score_raw_t<BF16>(q, rows, hq, hkv, batch, scale, head_reduce, scores, score_stride, stream);
   if (dtype == OKV_F16)
     return launch_score_raw_t<F16>(q, rows, hq, hkv, batch, scale, head_reduce, scores, score_stride, stream);
+  return false;
+}
+
+// The dense pass (contiguous 16-bit K/V, no index, no tail) with the query window riding along.
+bool launch_stage1_window(int dtype, const void* q, const RowList& rows, int hq, int hkv, int batch, float scale,
+                          const AttnWorkspace& w, const WindowFuse& wf, hipStream_t stream) {
+  if (rows.token_stride >= (1ll << 31) || rows.idx || rows.page_table || rows.max_tail_len != 0 || rows.tail_lens)
+    return false;
+  const int G = hq / hkv;
+  if (wf.window < 1 || wf.window * G > kWinCols) return false;
+#define OKV_WIN(T, GG) launch_one<T, GG, true, 0, false, true>(q, rows, hq, hkv, batch, scale, w, stream, wf)
+  if (dtype == OKV_BF16) {
+    switch (G) {
+      case 1: OKV_WIN(BF16, 1); return true;
+      case 2: OKV_WIN(BF16, 2); return true;
+      case 4: OKV_WIN(BF16, 4); return true;
+      case 8: OKV_WIN(BF16, 8); return true;
+    }
+  } else if (dtype == OKV_F16) {
+    switch (G) {
+      case 1: OKV_WIN(F16, 1); return true;
+      case 2: OKV_WIN(F16, 2); return true;
+      case 4: OKV_WIN(F16, 4); return true;
+      case 8: OKV_WIN(F16, 8); return true;
+    }
+  }
+#undef OKV_WIN
   return false;
 }
 

@@ -143,12 +143,23 @@ struct AttnWorkspace {
   int32_t logit_heads;   // rows of `logits` per request: Hq, or Hkv when group_reduce
 };
 
+// The last W query positions of every q head riding along a dense pass (window selectors): the
+// pass then also leaves, per scored split, the log-sum-exp of every (position, head) column's
+// logits, which is what the first of the window selector's two passes over K computes.
+constexpr int kWinCols = 64;  // columns (positions x q heads of one kv head) per kv head
+struct WindowFuse {
+  const void* wq;  // element (b, h, w, d) at wq + b*q_batch_stride + h*q_head_stride + w*q_pos_stride + d
+  int64_t q_batch_stride, q_head_stride, q_pos_stride;
+  int32_t window;
+  float* part;  // [batch][Hkv][kWinCols][max_splits]  log2-domain partial log-sum-exp
+};
+
 size_t attn_workspace_bytes(int batch, int hq, int hkv, int d, int max_main, int max_tail,
                             int max_score, bool with_v, bool with_logits,
-                            int* split_rows, int* max_splits, bool gather = false);
+                            int* split_rows, int* max_splits, int kind = 0);  // kind: 0 plain, 1 gather, 2 with a query window
 int carve_attn_workspace(void* ws, size_t ws_bytes, int batch, int hq, int hkv, int d,
                          int max_main, int max_tail, int max_score, bool with_v,
-                         bool with_logits, AttnWorkspace* out, bool gather = false);
+                         bool with_logits, AttnWorkspace* out, int kind = 0);
 
 extern std::atomic<int> g_split_rows_override;  // 0 = automatic
 
@@ -169,5 +180,10 @@ int launch_attention(const void* q, const RowList& rows, const okv_kv_layout_t* 
                      int batch, float scale, void* out, bool with_v, int head_reduce,
                      int normalise, float* scores, int64_t score_stride,
                      const AttnWorkspace& w, hipStream_t stream);
+
+int launch_attention_window(const void* q, const RowList& rows, const okv_kv_layout_t* layout, int batch,
+                            float scale, void* out, const AttnWorkspace& w, const WindowFuse& wf,
+                            hipStream_t stream);
+void fill_main(RowList* r, const void* k, const void* v, const okv_kv_layout_t* layout);
 
 }  // namespace okv

@@ -20,8 +20,6 @@
 
 namespace okv {
 
-constexpr int kWinCols = 64;  // columns (positions x q heads of one kv head) per kv head
-
 struct WindowArgs {
   const void* q;
   int64_t q_batch_stride, q_head_stride, q_pos_stride;  // elements
@@ -318,16 +316,19 @@ static int num_cus() {
   return 256;
 }
 
+static size_t window_part_bytes(int batch, int hkv, int splits);
+
 size_t window_workspace_bytes(int batch, int hkv, int max_len) {
   const int sr = window_split_rows(batch, hkv, max_len, num_cus());
   const int splits = (max_len + sr - 1) / sr;
-  return (size_t)batch * hkv * kWinCols * ((size_t)(splits > 0 ? splits : 1) + 1) * sizeof(float) + 512;
+  return window_part_bytes(batch, hkv, splits);
 }
 
 template <typename T, int NCB>
 static void launch_window(WindowArgs a, int batch, int exp_decay, float* scores, int64_t score_stride,
-                          int cus, hipStream_t stream) {
-  hipLaunchKernelGGL((window_lse_mfma<T, NCB>), dim3(a.hkv, a.max_splits, batch), dim3(256), 0, stream, a);
+                          int cus, hipStream_t stream, bool lse_parts_ready) {
+  if (!lse_parts_ready)  // otherwise the dense pass of the same call has left them
+    hipLaunchKernelGGL((window_lse_mfma<T, NCB>), dim3(a.hkv, a.max_splits, batch), dim3(256), 0, stream, a);
   hipLaunchKernelGGL(window_lse_merge, dim3(batch * a.hkv), dim3(256), 0, stream, a);
   // one round of row blocks, two blocks of `hkv` waves per CU; LDS bounds the rows
   int64_t per = ((int64_t)a.max_score_len * batch + 2 * cus - 1) / (2 * cus);
@@ -346,14 +347,26 @@ static void launch_window(WindowArgs a, int batch, int exp_decay, float* scores,
 
 template <typename T>
 static void launch_window_t(const WindowArgs& a, int batch, int exp_decay, float* scores,
-                            int64_t score_stride, int cus, hipStream_t stream) {
+                            int64_t score_stride, int cus, hipStream_t stream, bool lse_parts_ready = false) {
   const int ncb = (a.window * a.group + 15) / 16;
   switch (ncb) {
-    case 1: launch_window<T, 1>(a, batch, exp_decay, scores, score_stride, cus, stream); break;
-    case 2: launch_window<T, 2>(a, batch, exp_decay, scores, score_stride, cus, stream); break;
-    case 3: launch_window<T, 3>(a, batch, exp_decay, scores, score_stride, cus, stream); break;
-    default: launch_window<T, 4>(a, batch, exp_decay, scores, score_stride, cus, stream); break;
+    case 1: launch_window<T, 1>(a, batch, exp_decay, scores, score_stride, cus, stream, lse_parts_ready); break;
+    case 2: launch_window<T, 2>(a, batch, exp_decay, scores, score_stride, cus, stream, lse_parts_ready); break;
+    case 3: launch_window<T, 3>(a, batch, exp_decay, scores, score_stride, cus, stream, lse_parts_ready); break;
+    default: launch_window<T, 4>(a, batch, exp_decay, scores, score_stride, cus, stream, lse_parts_ready); break;
   }
+}
+
+// bytes of the window columns' partials and merged log-sum-exps for `splits` splits per request
+static size_t window_part_bytes(int batch, int hkv, int splits) {
+  return (size_t)batch * hkv * kWinCols * ((size_t)(splits > 0 ? splits : 1) + 1) * sizeof(float) + 512;
+}
+
+size_t dense_window_workspace_bytes(int batch, int hq, int hkv, int d, int max_seq_len, int max_score_len) {
+  int splits = 0;
+  const size_t attn = attn_workspace_bytes(batch, hq, hkv, d, max_seq_len, 0, max_score_len, true, false, nullptr,
+                                           &splits, 2);
+  return ((attn + 255) & ~(size_t)255) + window_part_bytes(batch, hkv, splits);
 }
 
 }  // namespace okv
@@ -412,6 +425,83 @@ extern "C" int okv_score_window(const void* q, int64_t q_batch_stride, int64_t q
     launch_window_t<BF16>(a, batch, exp_decay != 0, scores, score_stride, cus, (hipStream_t)stream);
   else
     launch_window_t<F16>(a, batch, exp_decay != 0, scores, score_stride, cus, (hipStream_t)stream);
+  OKV_HIP_CHECK(hipGetLastError());
+  return OKV_OK;
+}
+
+extern "C" int okv_dense_attn_window(const void* q, const void* q_window, int64_t q_batch_stride,
+                                     int64_t q_head_stride, int64_t q_pos_stride, int32_t window,
+                                     int32_t exp_decay, const void* k_base, const void* v_base,
+                                     const okv_kv_layout_t* layout, const int32_t* seq_lens, int32_t max_seq_len,
+                                     int32_t batch, float scale, void* out, const int32_t* score_lens,
+                                     int32_t max_score_len, float* scores, int64_t score_stride, void* ws,
+                                     size_t ws_bytes, okv_stream_t stream) {
+  int rc = validate_layout(layout, k_base, v_base);
+  if (rc) return rc;
+  OKV_REQUIRE(q && q_window && scores && out && v_base, OKV_ERR_INVALID, "q, q_window, v_base, out or scores is NULL");
+  OKV_REQUIRE(batch >= 1 && max_seq_len >= 1 && window >= 1, OKV_ERR_INVALID, "bad batch, length or window");
+  OKV_REQUIRE(max_score_len >= 1 && max_score_len <= max_seq_len, OKV_ERR_INVALID, "max_score_len out of range");
+  OKV_REQUIRE(score_stride >= max_score_len, OKV_ERR_INVALID, "score_stride < max_score_len");
+  OKV_REQUIRE(((uintptr_t)q_window & 15) == 0 && ((uintptr_t)q & 15) == 0 && q_batch_stride % 8 == 0 &&
+                  q_head_stride % 8 == 0 && q_pos_stride % 8 == 0,
+              OKV_ERR_INVALID, "q and q_window must be 16-byte aligned with strides that are multiples of 8");
+  const int hq = layout->num_q_heads, hkv = layout->num_kv_heads, group = hq / hkv;
+  OKV_REQUIRE(layout->dtype == OKV_BF16 || layout->dtype == OKV_F16, OKV_ERR_UNSUPPORTED,
+              "window scoring runs on the matrix cores: 16-bit K only");
+  OKV_REQUIRE(layout->page_table == nullptr, OKV_ERR_UNSUPPORTED, "window scoring reads contiguous K only");
+  OKV_REQUIRE(window * group <= kWinCols, OKV_ERR_UNSUPPORTED,
+              "window %d x group %d exceeds %d query rows per kv head", window, group, kWinCols);
+  OKV_REQUIRE(hkv <= 8, OKV_ERR_UNSUPPORTED, "more than 8 kv heads");
+  OKV_REQUIRE(layout->token_stride < (1ll << 31), OKV_ERR_UNSUPPORTED, "token stride too large");
+  const size_t need = dense_window_workspace_bytes(batch, hq, hkv, layout->head_dim, max_seq_len, max_score_len);
+  OKV_REQUIRE(ws != nullptr && ws_bytes >= need, OKV_ERR_WORKSPACE, "workspace too small: have %zu, need %zu",
+              ws_bytes, need);
+  const size_t attn_bytes = (attn_workspace_bytes(batch, hq, hkv, layout->head_dim, max_seq_len, 0, max_score_len,
+                                                  true, false, nullptr, nullptr, 2) + 255) & ~(size_t)255;
+  AttnWorkspace w;
+  rc = carve_attn_workspace(ws, attn_bytes, batch, hq, hkv, layout->head_dim, max_seq_len, 0, max_score_len, true,
+                            false, &w, 2);
+  if (rc) return rc;
+  WindowArgs a;
+  a.q = q_window;
+  a.q_batch_stride = q_batch_stride;
+  a.q_head_stride = q_head_stride;
+  a.q_pos_stride = q_pos_stride;
+  a.k_base = k_base;
+  a.token_stride = layout->token_stride;
+  a.head_stride = layout->head_stride;
+  a.batch_stride = layout->batch_stride;
+  a.score_lens = score_lens;
+  a.max_score_len = max_score_len;
+  a.window = window;
+  a.group = group;
+  a.hkv = hkv;
+  a.scale = scale;
+  a.split_rows = w.split_rows;  // the dense pass's splits: its scored ones tile [0, score_len)
+  a.max_splits = w.max_splits;
+  char* p = (char*)(((uintptr_t)ws + attn_bytes + 255) & ~(uintptr_t)255);
+  a.part = (float*)p;
+  a.lse = a.part + (size_t)batch * hkv * kWinCols * a.max_splits;
+  WindowFuse wf;
+  wf.wq = q_window;
+  wf.q_batch_stride = q_batch_stride;
+  wf.q_head_stride = q_head_stride;
+  wf.q_pos_stride = q_pos_stride;
+  wf.window = window;
+  wf.part = a.part;
+  RowList r;
+  fill_main(&r, k_base, v_base, layout);
+  r.main_lens = seq_lens;
+  r.max_main_len = max_seq_len;
+  r.score_lens = score_lens;
+  r.max_score_len = max_score_len;
+  rc = launch_attention_window(q, r, layout, batch, scale, out, w, wf, (hipStream_t)stream);
+  if (rc) return rc;
+  const int cus = num_cus();
+  if (layout->dtype == OKV_BF16)
+    launch_window_t<BF16>(a, batch, exp_decay != 0, scores, score_stride, cus, (hipStream_t)stream, true);
+  else
+    launch_window_t<F16>(a, batch, exp_decay != 0, scores, score_stride, cus, (hipStream_t)stream, true);
   OKV_HIP_CHECK(hipGetLastError());
   return OKV_OK;
 }

@@ -61,7 +61,8 @@ def main():
         trace.set_tracer(tracer)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    logits, cache = lm.forward(ids, None, max_new_tokens=args.steps + 16, offload_mode=args.offload_mode)
+    # room for the warm-up steps, and for the eager steps a window selector takes before a capture
+    logits, cache = lm.forward(ids, None, max_new_tokens=args.steps + 48, offload_mode=args.offload_mode)
     torch.cuda.synchronize()
     prefill_s = time.perf_counter() - t0
     tok = logits[:, -1].argmax(-1, keepdim=True)

@@ -25,7 +25,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--op", required=True,
                     choices=["dense", "fused", "fused_select", "fused_then_topk", "score", "topk", "sparse", "sparse_packed", "sparse_floor", "empty", "gather", "copy",
-                             "offload_memcpy", "offload_zero_copy", "offload_incremental", "h2d", "window", "window_loop",
+                             "offload_memcpy", "offload_zero_copy", "offload_incremental", "h2d", "window", "window_loop", "window_fused", "window_then_dense",
                              "paged_dense", "paged_fused", "paged_fused_select", "paged_score", "paged_topk", "paged_sparse", "paged_sparse_slots"])
     ap.add_argument("--batch", type=int, default=16, help="requests of the paged_* ops (ragged lengths 8192..32768)")
     ap.add_argument("--page-size", type=int, default=16)
@@ -157,6 +157,11 @@ def main():
             return ops.topk(scores, k_sel)
         if args.op == "window":
             return ops.score_window(qw[l], ks[l][:, :, :n], selector="uniform")
+        if args.op == "window_fused":  # a window-selector filter layer in two passes over K
+            return ops.dense_attn_window(qs[l], qw[l], ks[l], vs[l], selector="uniform", score_len=n)
+        if args.op == "window_then_dense":  # the same as two calls: three passes over K
+            ops.score_window(qw[l], ks[l][:, :, :n], selector="uniform")
+            return ops.dense_attn(qs[l], ks[l], vs[l])
         if args.op == "window_loop":
             acc = None
             for t in range(args.window):
@@ -191,6 +196,8 @@ def main():
         "score": 1.0 * n * row + 4.0 * n,
         "topk": 4.0 * n + 4.0 * k_sel,
         "window": 1.0 * n * row + 4.0 * n,  # one reading of K; the kernels read it twice
+        "window_fused": 2.0 * (n + tail) * row + 4.0 * n,  # one reading of K and V; K is read twice
+        "window_then_dense": 2.0 * (n + tail) * row + 4.0 * n,
         "window_loop": 1.0 * n * row + 4.0 * n,
         "sparse": 2.0 * (k_sel + tail) * row + 4.0 * k_sel,
         "sparse_packed": 2.0 * (k_sel + tail) * row,

@@ -237,9 +237,11 @@ class OmniKVMulLayer(nn.Module):
                     wq = attn.q_proj(win).view(win.shape[0], win.shape[1], attn.num_heads, attn.head_dim).transpose(1, 2)
                     cos, sin = attn.rotary_emb(wq, position_ids)
                     wq, _ = apply_rotary_pos_emb(wq, wq, cos, sin)
-                    past_key_value.select_with_query(wq.contiguous(), self.layer_idx, max(1, num_selected_tokens - forced),
-                                                     consider_len - forced, self.selector_cls, forced_tail=forced)
-                    o = past_key_value.attend(q, self.layer_idx)
+                    # the first of the two scoring passes over K rides on the layer's own attention
+                    o, _ = past_key_value.attend_and_select_window(q, wq.contiguous(), self.layer_idx,
+                                                                   max(1, num_selected_tokens - forced),
+                                                                   consider_len - forced, self.selector_cls,
+                                                                   forced_tail=forced)
                 past_key_value.stage = "decoding"
                 self.decode_step += 1
             else:

@@ -203,6 +203,46 @@ def score_window(q, k, score_len: Optional[int] = None, selector: str = "uniform
     return out
 
 
+def dense_attn_window(q, q_window, k, v, selector: str = "uniform", seq_len: Optional[int] = None,
+                      seq_lens: Optional[torch.Tensor] = None, score_len: Optional[int] = None,
+                      score_lens: Optional[torch.Tensor] = None, scale: Optional[float] = None,
+                      scores_out: Optional[torch.Tensor] = None):
+    """A window-selector filter layer in two passes over K: (out, scores) = (dense_attn(q, k, v),
+    score_window(q_window, k, score_len)) with the first scoring pass done inside the attention's;
+    okv_dense_attn_window.  q: (bsz, Hq, D) or (bsz, Hq, 1, D); q_window: (bsz, Hq, W, D), oldest first."""
+    q = _q3(q)
+    _require_gpu(q, "q")
+    _require_gpu(q_window, "q_window")
+    if selector not in ("uniform", "exp"):
+        raise ValueError(f"selector {selector!r} is not a window selector")
+    if q_window.dim() != 4 or q_window.stride(3) != 1 or q_window.dtype != q.dtype:
+        raise ValueError("q_window must be (bsz, Hq, W, D) with contiguous D and q's dtype")
+    hq, d = q.shape[1], q.shape[2]
+    if q_window.shape[0] != q.shape[0] or q_window.shape[1] != hq or q_window.shape[3] != d:
+        raise ValueError("q_window does not match q")
+    lay, kp, vp, batch, n = _layout(k, v, hq)
+    _same_dtype(q, lay)
+    if seq_len is None:
+        seq_len = n
+    if score_len is None:
+        score_len = seq_len
+    out = torch.empty_like(q)
+    scores = scores_out
+    if scores is None:
+        scores = torch.empty((batch, score_len), dtype=torch.float32, device=q.device)
+    elif scores.shape != (batch, score_len) or scores.dtype != torch.float32 or scores.stride(1) != 1:
+        raise ValueError("scores_out must be (bsz, score_len) float32 with contiguous rows")
+    nbytes = workspace_bytes(_lib.OKV_OP_DENSE_ATTN_WINDOW, batch, hq, lay.num_kv_heads, d, seq_len)
+    ws = _workspace(q.device, nbytes)
+    check(lib().okv_dense_attn_window(
+        q.data_ptr(), q_window.data_ptr(), q_window.stride(0), q_window.stride(1), q_window.stride(2),
+        q_window.shape[2], int(selector == "exp"), kp, vp, C.byref(lay), _lens(seq_lens, batch, "seq_lens"), seq_len,
+        batch, scale if scale is not None else 1.0 / math.sqrt(d), out.data_ptr(),
+        _lens(score_lens, batch, "score_lens"), score_len, scores.data_ptr(), scores.stride(0),
+        ws.data_ptr(), ws.numel(), _stream_ptr(q.device)))
+    return out, scores
+
+
 def topk(scores: torch.Tensor, k: int, seq_lens: Optional[torch.Tensor] = None,
          k_per_seg: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """(bsz, min(k, N)) int32 ascending indices of the k largest scores; okv_topk."""

@@ -414,6 +414,52 @@ def test_window_scores_ragged_batch_and_strided_q():
         assert torch.equal(got[b, :n], got_view[b, :n])
 
 
+@pytest.mark.parametrize("selector", ["uniform", "exp"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("w,hq,hkv,n,extra", [(16, 32, 8, 4099, 1), (16, 32, 8, 70001, 1), (16, 32, 8, 20000, 37),
+                                              (3, 32, 8, 4096, 1), (8, 32, 4, 3000, 5), (5, 8, 8, 2048, 1),
+                                              (7, 16, 8, 777, 0)])
+def test_window_filter_layer_in_two_passes(selector, dtype, w, hq, hkv, n, extra):
+    """okv_dense_attn_window: the layer's attention over n + extra rows and the window scores of the first
+    n from one call, against the oracle and against the two separate calls (the attention's pass over K
+    computes the window columns' log-sum-exps, grouped by its own splits)."""
+    q, k = _window_inputs(n + extra, w, hq, hkv, dtype)
+    g = torch.Generator().manual_seed(n + w)
+    v = torch.randn(k.shape, generator=g).to(dtype)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    q_last = qd[:, :, -1:].contiguous()
+    out, scores = ops.dense_attn_window(q_last, qd, kd, vd, selector=selector, score_len=n)
+    want_o = orc.gqa_attention(q[:, :, -1:].float(), k.float(), v.float())[:, :, 0, :]
+    want_s = orc.score_tokens(q.float(), k.float(), n, selector)
+    assert (out.cpu().float() - want_o).abs().max() < ATTN_TOL[dtype]
+    assert scores.shape == want_s.shape
+    assert _rel_err(scores.cpu(), want_s) < 1e-4
+    assert (out.float() - ops.dense_attn(q_last, kd, vd).float()).abs().max() < 1e-2
+    assert _rel_err(scores.cpu(), ops.score_window(qd, kd, score_len=n, selector=selector).cpu()) < 2e-5
+    kk = max(1, int(0.067 * n))
+    assert_near_tie_only(scores[0].cpu(), want_s[0], ops.topk(scores, kk).cpu()[0], orc.select_topk_stable(want_s, kk)[0], kk)
+
+
+def test_window_filter_layer_ragged_batch_static_shapes():
+    """Per-request lengths on the device, K/V buffers longer than any request (the captured decode
+    step's shapes), and an attention query that is not the window's last row."""
+    lens = [5000, 37, 2048, 640]
+    cap = 5200
+    qw, k = _window_inputs(cap, 16, 32, 8, torch.bfloat16, seed=33, bsz=4)
+    g = torch.Generator().manual_seed(34)
+    v = torch.randn(k.shape, generator=g).to(torch.bfloat16)
+    qa = torch.randn((4, 32, 1, 128), generator=g).to(torch.bfloat16)
+    seq = torch.tensor([n + 2 for n in lens], dtype=torch.int32, device=DEV)
+    sl = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    out, scores = ops.dense_attn_window(qa.to(DEV), qw.to(DEV), k.to(DEV), v.to(DEV), selector="uniform", seq_len=cap,
+                                        seq_lens=seq, score_len=5000, score_lens=sl)
+    for b, n in enumerate(lens):
+        want_o = orc.gqa_attention(qa[b:b + 1].float(), k[b:b + 1, :, :n + 2].float(), v[b:b + 1, :, :n + 2].float())[0, :, 0]
+        assert (out[b].cpu().float() - want_o).abs().max() < 2e-2, b
+        want_s = orc.score_tokens(qw[b:b + 1].float(), k[b:b + 1].float(), n, "uniform")
+        assert _rel_err(scores[b:b + 1, :n].cpu(), want_s) < 1e-4, b
+
+
 def test_window_unsupported_shapes_are_refused():
     q, k = _window_inputs(256, 17, 32, 8, torch.bfloat16)  # 17 positions x group 4 > 64 columns
     assert not ops.window_supported(q.to(DEV), k.to(DEV))
