@@ -112,7 +112,7 @@ int main() {
 
   // ---- one workspace for all calls: the largest any of them asks for
   size_t ws_bytes = 0;
-  for (int op : {OKV_OP_DENSE_ATTN, OKV_OP_TOPK, OKV_OP_SPARSE_ATTN}) {
+  for (int op : {OKV_OP_DENSE_ATTN, OKV_OP_TOPK, OKV_OP_SPARSE_ATTN, OKV_OP_DENSE_ATTN_SELECT, OKV_OP_DENSE_ATTN_WINDOW}) {
     okv_shape_t sh;
     std::memset(&sh, 0, sizeof(sh));
     sh.batch = 1;
@@ -205,6 +205,51 @@ int main() {
   std::vector<int> all(rows);
   std::iota(all.begin(), all.end(), 0);
   if (check_out(all, "dense attention") > 2e-2) return 8;
+
+  // ---- the filter layer as one call: the same three outputs, bit for bit
+  {
+    void* dout2;
+    float* dscores2;
+    int32_t* didx2;
+    HIP_OK(hipMalloc(&dout2, (size_t)HQ * D * 2));
+    HIP_OK(hipMalloc((void**)&dscores2, (size_t)N * 4));
+    HIP_OK(hipMalloc((void**)&didx2, (size_t)K_SEL * 4));
+    OKV(okv_dense_attn_select(dq, dk, dv, &lay, nullptr, N + T, 1, scale, dout2, nullptr, N, OKV_REDUCE_SUM,
+                              OKV_NORM_SOFTMAX, dscores2, N, nullptr, K_SEL, didx2, K_SEL, dws, ws_bytes, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    std::vector<float> scores2(N);
+    std::vector<int32_t> idx2(K_SEL);
+    std::vector<uint16_t> out2(HQ * D);
+    HIP_OK(hipMemcpy(scores2.data(), dscores2, (size_t)N * 4, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(idx2.data(), didx2, (size_t)K_SEL * 4, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(out2.data(), dout2, out2.size() * 2, hipMemcpyDeviceToHost));
+    if (std::memcmp(scores2.data(), scores.data(), (size_t)N * 4) != 0 || idx2 != idx || out2 != out) {
+      std::fprintf(stderr, "okv_dense_attn_select differs from okv_dense_attn + okv_topk\n");
+      return 12;
+    }
+    // ---- a window selector with a window of one position (the current query): per token the
+    // largest softmax probability over the heads; the attention is the same as above
+    OKV(okv_dense_attn_window(dq, dq, (int64_t)HQ * D, D, D, 1, 0, dk, dv, &lay, nullptr, N + T, 1, scale, dout2,
+                              nullptr, N, dscores2, N, dws, ws_bytes, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    HIP_OK(hipMemcpy(scores2.data(), dscores2, (size_t)N * 4, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(out2.data(), dout2, out2.size() * 2, hipMemcpyDeviceToHost));
+    std::vector<double> want_w(N, 0.0);
+    for (int h = 0; h < HQ; ++h) {
+      double m = -1e300, z = 0;
+      for (int t = 0; t < N; ++t) m = std::max(m, logit[h * rows + t]);
+      for (int t = 0; t < N; ++t) z += std::exp(logit[h * rows + t] - m);
+      for (int t = 0; t < N; ++t) want_w[t] = std::max(want_w[t], std::exp(logit[h * rows + t] - m) / z);
+    }
+    double ww = 0, wo = 0;
+    for (int t = 0; t < N; ++t) ww = std::max(ww, std::fabs(scores2[t] - want_w[t]) / (std::fabs(want_w[t]) + 1e-6));
+    for (int i = 0; i < HQ * D; ++i) wo = std::max(wo, (double)std::fabs(from_bf16(out2[i]) - from_bf16(out[i])));
+    std::printf("window filter layer: scores relative error %.3g, attention vs the dense call %.3g\n", ww, wo);
+    if (ww > 1e-3 || wo > 2e-2) return 13;
+    HIP_OK(hipFree(dout2));
+    HIP_OK(hipFree(dscores2));
+    HIP_OK(hipFree(didx2));
+  }
 
   // ---- sparse layer: the selected rows + the tail row (row N of the same buffers)
   const uint16_t* tk = (const uint16_t*)dk + (size_t)N * D;
