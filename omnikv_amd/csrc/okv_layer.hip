@@ -57,7 +57,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const T* __restrict__ x, c
   const T* xr = x + row * hidden;
   const T* rr = residual ? residual + row * hidden : nullptr;
   const bool vec = aligned16 && (hidden & 7) == 0 && hidden <= 256 * 8 * CH;
-  float h[CH][8];
+  float h[CH][8], wgt[CH][8];
   float ss = 0.f;
   if (vec) {
     float r[CH][8];
@@ -67,6 +67,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const T* __restrict__ x, c
       if (i < hidden) {
         ld8<T>(xr + i, h[c]);
         if (rr) ld8<T>(rr + i, r[c]);
+        ld8<T>(weight + i, wgt[c]);  // needed after the reduction only: one round trip instead of two
       }
     }
 #pragma unroll
@@ -103,10 +104,9 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const T* __restrict__ x, c
     for (int c = 0; c < CH; ++c) {
       const int i = (c * 256 + (int)threadIdx.x) * 8;
       if (i < hidden) {
-        float w[8], o[8];
-        ld8<T>(weight + i, w);
+        float o[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] = w[e] * rnd<T>(h[c][e] * rstd);
+        for (int e = 0; e < 8; ++e) o[e] = wgt[c][e] * rnd<T>(h[c][e] * rstd);
         st8<T>(out + row * hidden + i, o);
       }
     }
