@@ -607,13 +607,13 @@ int okv_dense_attn_select(const void* q, const void* k_base, const void* v_base,
   const size_t attn_bytes = (attn_workspace_bytes(batch, layout->num_q_heads, layout->num_kv_heads,
                                                   layout->head_dim, max_seq_len, 0, max_score_len, true, true,
                                                   nullptr, nullptr) + 255) & ~(size_t)255;
+  // long score vectors are selected by many workgroups, which need their own part of the workspace
+  const size_t need = attn_bytes + (max_score_len >= kMultiBlockMinLen ? topk_mb_workspace_bytes(batch, max_score_len) : 0);
   OKV_REQUIRE(ws != nullptr, OKV_ERR_INVALID, "workspace pointer is NULL");
-  OKV_REQUIRE(ws_bytes >= attn_bytes, OKV_ERR_WORKSPACE, "workspace too small: have %zu, need %zu", ws_bytes,
-              attn_bytes);
+  OKV_REQUIRE(ws_bytes >= need, OKV_ERR_WORKSPACE, "workspace too small: have %zu, need %zu", ws_bytes, need);
   int rc = okv_dense_attn(q, k_base, v_base, layout, seq_lens, max_seq_len, batch, scale, out, score_lens,
                           max_score_len, head_reduce, normalise, scores, score_stride, ws, attn_bytes, stream);
   if (rc) return rc;
-  // what is left of the workspace decides, as in okv_topk, whether long vectors get many workgroups
   return okv_topk(scores, score_stride, score_lens, max_score_len, k_per_seg, max_k, batch, idx_out, idx_stride,
                   (char*)ws + attn_bytes, ws_bytes - attn_bytes, stream);
 }

@@ -172,6 +172,7 @@ inline int finish_tokens_for(int split_rows, int max_score_len) {
 }
 
 size_t topk_mb_workspace_bytes(int batch, int max_seq_len);  // okv_topk_mb.hip
+static constexpr int kMultiBlockMinLen = 14336;  // top-k of shorter vectors: one workgroup per request is faster
 
 int validate_layout(const okv_kv_layout_t* layout, const void* k_base, const void* v_base);
 

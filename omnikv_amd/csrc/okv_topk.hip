@@ -17,7 +17,6 @@ static constexpr int kThreads = 1024;
 static constexpr int kWaves = kThreads / 64;
 static constexpr int kBins = 2048;
 static constexpr int kCandCap = 8192;  // candidate keys held in LDS (32 KB)
-static constexpr int kMultiBlockMinLen = 14336;  // below this one workgroup per request is faster
 
 __device__ __forceinline__ uint32_t score_key(float s) {
   uint32_t u = __float_as_uint(s);

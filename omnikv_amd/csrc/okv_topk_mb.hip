@@ -63,13 +63,20 @@ static void chunking(int max_seq_len, int* chunk_tiles, int* chunks) {
 
 static inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
+// An upper bound of what carve_topk() lays out that never shrinks when max_seq_len grows (the
+// exact layout does, where one more tile makes the chunks twice as long and half as many), so
+// that a workspace sized for a length also serves every shorter one.
 size_t topk_mb_workspace_bytes(int batch, int max_seq_len) {
-  int ct, chunks;
-  chunking(max_seq_len, &ct, &chunks);
+  const int tiles = (max_seq_len + kTile - 1) / kTile;
+  int chunks = tiles < kTargetChunks ? tiles : kTargetChunks;            // chunks of up to kMaxChunkTiles tiles: at most
+  const int long_chunks = (tiles + kMaxChunkTiles - 1) / kMaxChunkTiles;  // this many, or that many once they are full
+  if (long_chunks > chunks) chunks = long_chunks;
+  if (chunks < 1) chunks = 1;
+  const size_t cand_tiles = (size_t)tiles + kMaxChunkTiles;  // chunks * tiles per chunk < tiles + tiles per chunk
   size_t b = 0;
   b += up256((size_t)batch * chunks * kBins12 * 2);
   b += up256((size_t)batch * chunks * 256 * 2);
-  b += up256((size_t)batch * chunks * ct * kTile * 4);
+  b += up256((size_t)batch * cand_tiles * kTile * 4);
   b += up256((size_t)batch * chunks * 4);
   b += up256((size_t)batch * chunks * kMbWaves * 4);
   b += up256((size_t)batch * sizeof(TopkMbState));

@@ -180,6 +180,22 @@ def test_filter_layer_in_one_call_equals_attention_then_topk(selector, dtype, n,
     assert torch.equal(idx1.cpu().to(torch.int64), want)
 
 
+def test_filter_layer_in_one_call_where_the_topk_chunking_changes():
+    """262145 rows attended, 262144 scored: the workspace is sized by the attention's length, whose top-k
+    would use 33 chunks of two tiles, while the scores' own length makes 64 chunks of one."""
+    n = 64 * 4096
+    g = torch.Generator().manual_seed(5)
+    k = torch.randn((1, 8, n + 1, 128), generator=g).to(torch.bfloat16).to(DEV)
+    v = torch.randn((1, 8, n + 1, 128), generator=g).to(torch.bfloat16).to(DEV)
+    q = torch.randn((1, 32, 1, 128), generator=g).to(torch.bfloat16).to(DEV)
+    ksel = int(0.067 * n)
+    out2, scores2 = ops.dense_attn(q, k, v, selector="softmax_sum_last", score_len=n)
+    out1, scores1, idx1 = ops.dense_attn(q, k, v, selector="softmax_sum_last", score_len=n, select_k=ksel)
+    assert torch.equal(out1, out2) and torch.equal(scores1, scores2)
+    assert torch.equal(idx1, ops.topk(scores2, ksel))
+    assert torch.equal(idx1.cpu().to(torch.int64), orc.select_topk_stable(scores1.cpu(), ksel))
+
+
 def test_filter_layer_in_one_call_ragged_batch_and_both_block_sizes():
     """Requests of different lengths (one empty, one shorter than a score-finishing block, two ending
     inside one) with per-request k, at the automatic split size and at one small enough that the

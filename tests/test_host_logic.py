@@ -107,6 +107,19 @@ def test_workspace_sizes_are_consistent():
     big = ops.workspace_bytes(_lib.OKV_OP_SPARSE_ATTN, 16, 32, 8, 128, 2195, 64)
     assert 0 < small < big
     assert ops.workspace_bytes(_lib.OKV_OP_TOPK, 1, 0, 0, 0, 450000) > 0
+    # a workspace sized for a length serves every shorter one: the top-k's size never shrinks as the length
+    # grows (its chunks become twice as long and half as many at 64 * 4096 + 1 scores), and the one-call filter
+    # layer, sized by the attention's length, covers the attention's and the top-k's parts at any score length
+    lengths = sorted(list(range(1, 700000, 4093)) + [262144, 262145, 4096 * 960, 4096 * 960 + 1, 5000000])
+    for b in (1, 16):
+        run = [ops.workspace_bytes(_lib.OKV_OP_TOPK, b, 0, 0, 0, n) for n in lengths]
+        assert all(y >= x for x, y in zip(run, run[1:]))
+    for n in (4096, 131073, 262145, 450001):
+        both = ops.workspace_bytes(_lib.OKV_OP_DENSE_ATTN_SELECT, 1, 32, 8, 128, n)
+        assert both >= ops.workspace_bytes(_lib.OKV_OP_DENSE_ATTN, 1, 32, 8, 128, n, with_scores=True) - 512 + \
+            ops.workspace_bytes(_lib.OKV_OP_TOPK, 1, 0, 0, 0, n - 1)
+    win = ops.workspace_bytes(_lib.OKV_OP_DENSE_ATTN_WINDOW, 1, 32, 8, 128, 131073)
+    assert win > ops.workspace_bytes(_lib.OKV_OP_DENSE_ATTN, 1, 32, 8, 128, 131073) // 4
     out = C.c_size_t(0)
     assert _lib.lib().okv_workspace_bytes(99, C.byref(_lib.Shape(1, 32, 8, 128, 10, 0, 0)), C.byref(out)) == -1
     assert _lib.lib().okv_workspace_bytes(0, None, C.byref(out)) == -1
