@@ -6,15 +6,18 @@
 // 32s + 8(l/16) .. +8 of k-step s -- loaded in that layout by the gather modes, loaded as
 // whole streamed rows and turned into it through LDS by the streaming modes; the G q
 // heads of the kv head are the first G columns of the B operand, the rest zero).  The result leaves
-// lane l holding column (head) l%16 of tile rows 4(l/16) .. +4: the lanes of one
-// 16-lane row hold all heads of the same four rows, so each row of lanes keeps its
-// own online softmax, and the probabilities reach the P.V lanes by DPP row
-// broadcasts.  P.V is VALU work on packed pairs: lane l owns output elements
-// 8(l%16) .. +8 and accumulates the four rows of its lane row with v_dot2 (two rows
-// per instruction, probabilities rounded to the K/V element type as matrix-core
-// attention does), reading V fully coalesced (256 bytes per row per 16 lanes).
+// lane l holding column (head) l%16 of tile rows 4(l/16) .. +4 -- which is the A-operand
+// layout of v_mfma_f32_16x16x16 with the heads as rows and the tile's 16 rows as the
+// contraction.  So P.V runs on the matrix cores too: the probabilities, rounded to the K/V
+// element type, are the A operand as they stand, and V, read fully coalesced as whole rows
+// (256 bytes per row per 16 lanes: lane l holds elements 8(l%16) .. +8 of rows 4(l/16) .. +4),
+// gives eight B operands, one per element position e (column n of block e is output element
+// 8n + e), after sixteen v_perm that pair the rows.  The wave keeps ONE running maximum per
+// head (a tile whose logits stay below it costs a compare and a ballot; one that raises it,
+// two lane-row exchanges and a rescale of the accumulators), so the four waves of the block,
+// not sixteen lane rows, meet in LDS at the end.
 // The rows of tile t+2 are looked up and the K/V of tile t+1 are in flight while
-// tile t is consumed.  The sixteen lane rows of the block meet in LDS at the end.
+// tile t is consumed.
 #include <math.h>
 
 #include <atomic>
@@ -33,14 +36,19 @@ __device__ __forceinline__ uint32_t pack2(const F16*, float a, float b) {
   f32x2_t x = {a, b};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2_t));
 }
-// acc + v.lo*p.lo + v.hi*p.hi
-__device__ __forceinline__ float dot2(const BF16*, uint32_t v, uint32_t p, float acc) {
-  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, v),
-                                         __builtin_bit_cast(bf16x2_t, p), acc, false);
+// D(16 heads x 16 columns) += A(16 heads x 16 rows) . B(16 rows x 16 columns): lane l holds A row
+// l%16 / B column l%16, contraction elements 4(l/16) .. +4, and D column l%16, rows 4(l/16) .. +4.
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4_t;
+__device__ __forceinline__ f32x4_t mfma16k16(const BF16*, uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, f32x4_t c) {
+  const uint2 a = make_uint2(a0, a1), b = make_uint2(b0, b1);
+  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, a), __builtin_bit_cast(s16x4_t, b), c,
+                                                   0, 0, 0);
 }
-__device__ __forceinline__ float dot2(const F16*, uint32_t v, uint32_t p, float acc) {
-  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, v), __builtin_bit_cast(f16x2_t, p), acc,
-                                false);
+__device__ __forceinline__ f32x4_t mfma16k16(const F16*, uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, f32x4_t c) {
+  const uint2 a = make_uint2(a0, a1), b = make_uint2(b0, b1);
+  return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a), __builtin_bit_cast(f16x4_t, b), c, 0,
+                                               0, 0);
 }
 
 // value of lane H of the caller's 16-lane row
@@ -48,28 +56,41 @@ template <int H>
 __device__ __forceinline__ uint32_t row_bcast(uint32_t x) {
   return (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, 0x150 + H, 0xf, 0xf, true);
 }
+template <int H>
+__device__ __forceinline__ float row_bcast_f(float x) {
+  return __uint_as_float(row_bcast<H>(__float_as_uint(x)));
+}
 
-template <typename T, int H, int G>
-struct HeadStep {
-  // acc[h][:] += P_h(row pair) . V(row pair) for heads H .. G-1
-  static __device__ __forceinline__ void pv(float (&acc)[G][8], uint32_t p, const uint32_t (&vp)[8]) {
-    const uint32_t ph = row_bcast<H>(p);
+// max / sum over the four lane rows (lanes l, l^16, l^32, l^48), left in all of them
+__device__ __forceinline__ float lane_rows_max(float x) {
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float lane_rows_sum(float x) {
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+// The P.V accumulators of a wave: acc[e][i] of lane l is output element 8(l%16) + e of head
+// 4(l/16) + i.  Heads beyond G (lane rows beyond G/4) accumulate the zero-query columns and are
+// never read.
+template <int G>
+__device__ __forceinline__ void scale_heads(f32x4_t (&acc)[8], float alpha, int j4) {
+  float a[4] = {row_bcast_f<0>(alpha), row_bcast_f<1>(alpha), row_bcast_f<2>(alpha), row_bcast_f<3>(alpha)};
+  if (G > 4) {
+    const float b[4] = {row_bcast_f<4>(alpha), row_bcast_f<5>(alpha), row_bcast_f<6>(alpha), row_bcast_f<7>(alpha)};
 #pragma unroll
-    for (int d = 0; d < 8; ++d) acc[H][d] = dot2((const T*)nullptr, vp[d], ph, acc[H][d]);
-    HeadStep<T, H + 1, G>::pv(acc, p, vp);
+    for (int i = 0; i < 4; ++i) a[i] = (j4 & 1) ? b[i] : a[i];
   }
-  static __device__ __forceinline__ void scale(float (&acc)[G][8], float a) {
-    const float ah = __uint_as_float(row_bcast<H>(__float_as_uint(a)));
 #pragma unroll
-    for (int d = 0; d < 8; ++d) acc[H][d] *= ah;
-    HeadStep<T, H + 1, G>::scale(acc, a);
-  }
-};
-template <typename T, int G>
-struct HeadStep<T, G, G> {
-  static __device__ __forceinline__ void pv(float (&)[G][8], uint32_t, const uint32_t (&)[8]) {}
-  static __device__ __forceinline__ void scale(float (&)[G][8], float) {}
-};
+  for (int e = 0; e < 8; ++e)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[e][i] *= a[i];
+}
 
 // What a lane needs to know about the rows of a tile before it can address them:
 // the K row (index 0) and its four V rows (1..4).
@@ -80,7 +101,7 @@ struct TileRows {
 
 template <int G>
 __host__ __device__ constexpr int stage1_lds_floats(bool with_v) {
-  return 3 * 16 * G + 16 + (with_v ? 16 * G * kD : 0);
+  return 2 * 4 * G + 8 + (with_v ? 4 * G * kD : 0);  // per wave and head: max, sum, partial output
 }
 constexpr int kWindowLdsFloats = 2 * 16 * kWinCols;  // [16 lane rows][64 columns] running max and sum
 
@@ -232,12 +253,11 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
     }
   };
 
-  float m = -INFINITY, l = 0.f;  // softmax state of (head r16, lane row j4); m in raw q.k units
-  float acc[G][8];               // output elements 8*r16.. summed over the rows of lane row j4
+  float m = -INFINITY;  // running max of head r16 over the wave's rows so far (the same in all four lane rows); raw q.k units
+  float l = 0.f;        // sum of exp over the rows of lane row j4, relative to m
+  f32x4_t acc[8];       // acc[e][i]: output element 8*r16 + e of head 4*j4 + i, summed over the wave's rows
 #pragma unroll
-  for (int h = 0; h < G; ++h)
-#pragma unroll
-    for (int d = 0; d < 8; ++d) acc[h][d] = 0.f;
+  for (int e = 0; e < 8; ++e) acc[e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   const float sl2 = scale * kLog2e;
   const bool scored = LOGITS && begin < A;  // a scored split ends at or before A
   float* slog = lds;  // [G][split_rows] scaled logits of the split; flushed before LDS is reused below
@@ -308,40 +328,36 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
       for (int i = 0; i < 4; ++i)
         if (row0 + i >= end) s[i] = -INFINITY;
     }
-    const float mn = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), m);
-    const float ms = (partial && mn == -INFINITY) ? 0.f : mn;
-    const float neg = -ms * sl2;
-    const float alpha = __builtin_amdgcn_exp2f((m - ms) * sl2);  // exactly 1 while the max stands
+    const float ml = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
+    if (__ballot(ml > m) != 0ull) {  // some head's max moves (always on the wave's first tile)
+      const float mn = lane_rows_max(fmaxf(ml, m));
+      const float alpha = __builtin_amdgcn_exp2f((m - (mn == -INFINITY ? 0.f : mn)) * sl2);  // 1 for a head whose max stands
+      l *= alpha;
+      if (WITH_V) scale_heads<G>(acc, alpha, j4);
+      m = mn;
+    }
+    const float neg = (m == -INFINITY ? 0.f : -m) * sl2;
     float p[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) p[i] = __builtin_amdgcn_exp2f(fmaf(s[i], sl2, neg));
-    l = fmaf(l, alpha, (p[0] + p[1]) + (p[2] + p[3]));
-    const bool changed = (r16 < G) && (mn > m);
-    m = mn;
+    l += (p[0] + p[1]) + (p[2] + p[3]);
     if (WITH_V) {
-      if (__ballot(changed) != 0ull) HeadStep<T, 0, G>::scale(acc, alpha);
+      // A operand: P of head r16, rows 4*j4 .. +4, as it stands.  B operand of block e: element e of
+      // the lane's four V rows.
       const uint32_t p01 = pack2((const T*)nullptr, p[0], p[1]);
       const uint32_t p23 = pack2((const T*)nullptr, p[2], p[3]);
-      uint32_t vp[8];
-      {
-        const uint32_t a[4] = {vf[0].x, vf[0].y, vf[0].z, vf[0].w};
-        const uint32_t c[4] = {vf[1].x, vf[1].y, vf[1].z, vf[1].w};
+      const uint32_t a[4] = {vf[0].x, vf[0].y, vf[0].z, vf[0].w};
+      const uint32_t c[4] = {vf[1].x, vf[1].y, vf[1].z, vf[1].w};
+      const uint32_t x[4] = {vf[2].x, vf[2].y, vf[2].z, vf[2].w};
+      const uint32_t y[4] = {vf[3].x, vf[3].y, vf[3].z, vf[3].w};
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          vp[2 * j] = __builtin_amdgcn_perm(c[j], a[j], 0x05040100u);
-          vp[2 * j + 1] = __builtin_amdgcn_perm(c[j], a[j], 0x07060302u);
-        }
-        HeadStep<T, 0, G>::pv(acc, p01, vp);
-      }
-      {
-        const uint32_t a[4] = {vf[2].x, vf[2].y, vf[2].z, vf[2].w};
-        const uint32_t c[4] = {vf[3].x, vf[3].y, vf[3].z, vf[3].w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          vp[2 * j] = __builtin_amdgcn_perm(c[j], a[j], 0x05040100u);
-          vp[2 * j + 1] = __builtin_amdgcn_perm(c[j], a[j], 0x07060302u);
-        }
-        HeadStep<T, 0, G>::pv(acc, p23, vp);
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t lo01 = __builtin_amdgcn_perm(c[j], a[j], 0x05040100u);
+        const uint32_t hi01 = __builtin_amdgcn_perm(c[j], a[j], 0x07060302u);
+        const uint32_t lo23 = __builtin_amdgcn_perm(y[j], x[j], 0x05040100u);
+        const uint32_t hi23 = __builtin_amdgcn_perm(y[j], x[j], 0x07060302u);
+        acc[2 * j] = mfma16k16((const T*)nullptr, p01, p23, lo01, lo23, acc[2 * j]);
+        acc[2 * j + 1] = mfma16k16((const T*)nullptr, p01, p23, hi01, hi23, acc[2 * j + 1]);
       }
     }
   };
@@ -422,21 +438,25 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
     __syncthreads();
   }
 
-  // ---- the 16 lane rows of the block meet in LDS
-  float* sm = lds;                // [16][G] running max (raw units)
-  float* sl = lds + 16 * G;       // [16][G] sum of exp
-  float* sacc = lds + 48 * G + 16;  // [16][G][128]
+  // ---- the four waves of the block meet in LDS
+  float* sm = lds;                 // [4][G] running max (raw units)
+  float* sl = lds + 4 * G;         // [4][G] sum of exp
+  float* sacc = lds + 8 * G + 8;   // [4][G][128]
   const int grp = wave * 4 + j4;
-  if (r16 < G) {
-    sm[grp * G + r16] = m;
-    sl[grp * G + r16] = l;
+  l = lane_rows_sum(l);
+  if (r16 < G && j4 == 0) {
+    sm[wave * G + r16] = m;
+    sl[wave * G + r16] = l;
   }
   if (WITH_V) {
 #pragma unroll
-    for (int h = 0; h < G; ++h) {
-      float4* dst = reinterpret_cast<float4*>(sacc + (grp * G + h) * kD + r16 * 8);
-      dst[0] = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
-      dst[1] = make_float4(acc[h][4], acc[h][5], acc[h][6], acc[h][7]);
+    for (int i = 0; i < 4; ++i) {
+      const int h = 4 * j4 + i;
+      if (h < G) {
+        float4* dst = reinterpret_cast<float4*>(sacc + (wave * G + h) * kD + r16 * 8);
+        dst[0] = make_float4(acc[0][i], acc[1][i], acc[2][i], acc[3][i]);
+        dst[1] = make_float4(acc[4][i], acc[5][i], acc[6][i], acc[7][i]);
+      }
     }
   }
   if (WINDOW) {
@@ -470,10 +490,10 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
     const int h = o / kD, d = o % kD;
     float M = -INFINITY;
 #pragma unroll
-    for (int x = 0; x < 16; ++x) M = fmaxf(M, sm[x * G + h]);
+    for (int x = 0; x < 4; ++x) M = fmaxf(M, sm[x * G + h]);
     float den = 0.f, num = 0.f;
 #pragma unroll
-    for (int x = 0; x < 16; ++x) {
+    for (int x = 0; x < 4; ++x) {
       const float mm = sm[x * G + h];
       const float fx = (mm == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((mm - M) * sl2);
       den = fmaf(sl[x * G + h], fx, den);
