@@ -97,7 +97,15 @@ __device__ __forceinline__ void scale_heads(f32x4_t (&acc)[8], float alpha, int 
 struct TileRows {
   int32_t tok[5];  // token (or page) the row maps to; raw load results
   int32_t row[5];  // logical row, clamped into the split
+  bool direct;     // wave-uniform: all 16 rows are selected rows of the split -- tok[0] is the token of row
+                   // r16 (the lane's K row), tok[1] that of row 4*j4 + r16%4 (its quad holds the four V rows)
 };
+
+// value of lane I of the caller's quad
+template <int I>
+__device__ __forceinline__ uint32_t quad_bcast(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, I * 0x55, 0xf, 0xf, true);
+}
 
 template <int G>
 __host__ __device__ constexpr int stage1_lds_floats(bool with_v) {
@@ -129,19 +137,18 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
   rl_split_range(split, w.split_rows, A, L, &begin, &end);
   if (begin >= end) return;
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: tile bases and the paths below are wave-uniform
   const int r16 = lane & 15, j4 = lane >> 4;
 
-  // B operand: q heads of this kv head in columns 0..G-1, zero beyond
+  // B operand: q heads of this kv head in columns 0..G-1; the columns beyond repeat head G-1 (their
+  // results are never read, and unconditional loads keep the prologue free of branches)
   uint4 qf[4];
   {
     const int hcol = r16 < G ? r16 : G - 1;
     const T* qp = q + ((int64_t)(b * hq + g * G + hcol) * kD + 8 * j4);
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const uint4 v = *reinterpret_cast<const uint4*>(qp + 32 * s);
-      qf[s] = r16 < G ? v : make_uint4(0, 0, 0, 0);
-    }
+    for (int s = 0; s < 4; ++s) qf[s] = *reinterpret_cast<const uint4*>(qp + 32 * s);
   }
 
   constexpr int WCB = WINDOW ? kWinCols / 16 : 1;
@@ -182,7 +189,27 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
 
   // ---- which rows a tile touches (issues the index / page-table loads)
   const int32_t* idx_row = rows.idx + (int64_t)b * rows.idx_stride;
+  // Gather mode: two index loads per lane and tile -- the lane's K row (tile row r16) and one of its lane
+  // row's four V rows (tile row 4*j4 + r16%4; a quad holds the four between its lanes).  Both are always
+  // issued from clamped positions, so every tile has the same loads in flight; a row of the tail
+  // segment is carried as the complement of its position there (negative).  Tiles that lie wholly
+  // inside the selected rows of the split take the short address arithmetic.
+  const int direct_end = MODE == 1 ? min(main_len, end) : 0;
+  auto gather_tok = [&](int r) -> int32_t {
+    r = r < last ? r : last;
+    int ri = r < main_len ? r : main_len - 1;
+    ri = ri < 0 ? 0 : ri;  // a request with tail rows only: the index still holds one entry
+    const int32_t t = idx_row[ri];
+    const int32_t in_tail = (main_len - 1 - r) >> 31;  // all ones for a tail row
+    return t ^ ((t ^ ~(r - main_len)) & in_tail);
+  };
   auto tile_rows = [&](int tbase, TileRows& tr) {
+    if (MODE == 1) {
+      tr.direct = __builtin_amdgcn_readfirstlane(tbase) + 16 <= direct_end;
+      tr.tok[0] = gather_tok(tbase + r16);
+      tr.tok[1] = gather_tok(tbase + 4 * j4 + (r16 & 3));
+      return;
+    }
 #pragma unroll
     for (int x = 0; x < 5; ++x) {
       int r = x == 0 ? tbase + r16 : tbase + 4 * j4 + (x - 1);
@@ -200,11 +227,6 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
         } else {
           tr.tok[x] = rows.page_table[(int64_t)b * rows.page_table_stride + (r >> rows.page_shift)];
         }
-      } else if (MODE == 1) {  // branch-free: the index holds at least one entry per request
-        int ri = r < main_len ? r : main_len - 1;
-        ri = ri < 0 ? 0 : ri;  // a request with tail rows only
-        const int t = idx_row[ri];
-        tr.tok[x] = r < main_len ? t : r - main_len;
       } else if (r >= main_len) {
         tr.tok[x] = r - main_len;
       } else {
@@ -222,11 +244,6 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
     if (MODE == 3)
       return (is_v ? pvb : pkb) + (int64_t)tr.tok[x] * rows.page_stride +
              (uint64_t)(uint32_t)(tr.row[x] & (rows.page_size - 1)) * ts;
-    if (MODE == 1) {
-      const bool in_tail = tr.row[x] >= main_len;
-      const T* base = in_tail ? (is_v ? tvb : tkb) : (is_v ? vb : kb);
-      return base + (uint64_t)(uint32_t)tr.tok[x] * (in_tail ? tts : ts);
-    }
     if (tr.row[x] >= main_len) return (is_v ? tvb : tkb) + (uint64_t)(uint32_t)tr.tok[x] * tts;
     if (tr.row[x] < 0)
       return (is_v ? pvb : pkb) + (int64_t)tr.tok[x] * rows.page_stride +
@@ -234,6 +251,34 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
     return (is_v ? vb : kb) + (uint64_t)(uint32_t)tr.tok[x] * ts;
   };
   auto load_tile = [&](const TileRows& tr, uint4 (&kf)[4], uint4 (&vf)[4]) {
+    if (MODE == 1) {
+      // a row's address from its (possibly complemented) token: selected rows of K / V, or rows of the tail
+      auto addr = [&](int32_t e, bool is_v) -> const T* {
+        const bool in_tail = e < 0;
+        const uint32_t t = in_tail ? ~e : e;
+        return (in_tail ? (is_v ? tvb : tkb) : (is_v ? vb : kb)) + (uint64_t)t * (in_tail ? tts : ts);
+      };
+      const int32_t e4[4] = {(int32_t)quad_bcast<0>(tr.tok[1]), (int32_t)quad_bcast<1>(tr.tok[1]),
+                             (int32_t)quad_bcast<2>(tr.tok[1]), (int32_t)quad_bcast<3>(tr.tok[1])};
+      if (tr.direct) {  // wave-uniform: no tail row in the tile
+        const T* kp = kb + (uint64_t)(uint32_t)tr.tok[0] * ts + 8 * j4;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) kf[s] = *reinterpret_cast<const uint4*>(kp + 32 * s);
+        if (WITH_V) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) vf[i] = load_stream16(vb + (uint64_t)(uint32_t)e4[i] * ts + 8 * r16);
+        }
+      } else {
+        const T* kp = addr(tr.tok[0], false) + 8 * j4;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) kf[s] = *reinterpret_cast<const uint4*>(kp + 32 * s);
+        if (WITH_V) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) vf[i] = load_stream16(addr(e4[i], true) + 8 * r16);
+        }
+      }
+      return;
+    }
     if (KLDS) {
       // whole rows, like V; compute() turns the tile into the A-operand layout through LDS
 #pragma unroll
@@ -269,6 +314,7 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
   if (WINDOW) kst_off += kWindowLdsFloats;
   char* kstage = reinterpret_cast<char*>(lds + kst_off) + wave * 4096;
   auto compute = [&](int tbase, const uint4 (&kf_in)[4], const uint4 (&vf)[4]) {
+    float s[4];
     uint4 kf[4];
     if (KLDS) {
       k_rows_to_a_operand(kstage, r16, j4, kf_in, kf);
@@ -322,7 +368,8 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
         *reinterpret_cast<float4*>(slog + r16 * w.split_rows + (row0 - begin)) =
             make_float4(v[0], v[1], v[2], v[3]);
     }
-    float s[4] = {S[0], S[1], S[2], S[3]};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s[i] = S[i];
     if (partial) {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
@@ -333,7 +380,7 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
       const float mn = lane_rows_max(fmaxf(ml, m));
       const float alpha = __builtin_amdgcn_exp2f((m - (mn == -INFINITY ? 0.f : mn)) * sl2);  // 1 for a head whose max stands
       l *= alpha;
-      if (WITH_V) scale_heads<G>(acc, alpha, j4);
+      if (WITH_V) scale_heads<G>(acc, alpha, j4);  // nothing accumulated yet on the first tile
       m = mn;
     }
     const float neg = (m == -INFINITY ? 0.f : -m) * sl2;
@@ -342,41 +389,44 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
     for (int i = 0; i < 4; ++i) p[i] = __builtin_amdgcn_exp2f(fmaf(s[i], sl2, neg));
     l += (p[0] + p[1]) + (p[2] + p[3]);
     if (WITH_V) {
-      // A operand: P of head r16, rows 4*j4 .. +4, as it stands.  B operand of block e: element e of
-      // the lane's four V rows.
-      const uint32_t p01 = pack2((const T*)nullptr, p[0], p[1]);
-      const uint32_t p23 = pack2((const T*)nullptr, p[2], p[3]);
-      const uint32_t a[4] = {vf[0].x, vf[0].y, vf[0].z, vf[0].w};
-      const uint32_t c[4] = {vf[1].x, vf[1].y, vf[1].z, vf[1].w};
-      const uint32_t x[4] = {vf[2].x, vf[2].y, vf[2].z, vf[2].w};
-      const uint32_t y[4] = {vf[3].x, vf[3].y, vf[3].z, vf[3].w};
+    // A operand: P of head r16, rows 4*j4 .. +4, as it stands.  B operand of block e: element e of
+    // the lane's four V rows.
+    const uint32_t p01 = pack2((const T*)nullptr, p[0], p[1]);
+    const uint32_t p23 = pack2((const T*)nullptr, p[2], p[3]);
+    const uint32_t a[4] = {vf[0].x, vf[0].y, vf[0].z, vf[0].w};
+    const uint32_t c[4] = {vf[1].x, vf[1].y, vf[1].z, vf[1].w};
+    const uint32_t x[4] = {vf[2].x, vf[2].y, vf[2].z, vf[2].w};
+    const uint32_t y[4] = {vf[3].x, vf[3].y, vf[3].z, vf[3].w};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint32_t lo01 = __builtin_amdgcn_perm(c[j], a[j], 0x05040100u);
-        const uint32_t hi01 = __builtin_amdgcn_perm(c[j], a[j], 0x07060302u);
-        const uint32_t lo23 = __builtin_amdgcn_perm(y[j], x[j], 0x05040100u);
-        const uint32_t hi23 = __builtin_amdgcn_perm(y[j], x[j], 0x07060302u);
-        acc[2 * j] = mfma16k16((const T*)nullptr, p01, p23, lo01, lo23, acc[2 * j]);
-        acc[2 * j + 1] = mfma16k16((const T*)nullptr, p01, p23, hi01, hi23, acc[2 * j + 1]);
-      }
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t lo01 = __builtin_amdgcn_perm(c[j], a[j], 0x05040100u);
+      const uint32_t hi01 = __builtin_amdgcn_perm(c[j], a[j], 0x07060302u);
+      const uint32_t lo23 = __builtin_amdgcn_perm(y[j], x[j], 0x05040100u);
+      const uint32_t hi23 = __builtin_amdgcn_perm(y[j], x[j], 0x07060302u);
+      acc[2 * j] = mfma16k16((const T*)nullptr, p01, p23, lo01, lo23, acc[2 * j]);
+      acc[2 * j + 1] = mfma16k16((const T*)nullptr, p01, p23, hi01, hi23, acc[2 * j + 1]);
+    }
     }
   };
-
   // ---- tiles of this wave: begin + 16*(wave + 4*n).  Inside the loop every load is
   // unconditional (a tile index past the wave's last tile is clamped to it), so the
   // number of loads in flight is the same on every path and the wait before a tile's
   // first use leaves the next tile's loads outstanding.
   {
-    uint4 kA[4], vA[4], kB[4], vB[4];
-    TileRows tr, tr0;
     int t = begin + wave * 16;
     if (t < end) {
       const int t_last = t + ((last - t) >> 6 << 6);
-      tile_rows(t, tr0);
+      // every path issues all its first lookups before it waits for any of them
       if (t == t_last) {  // one tile
+        uint4 kA[4], vA[4];
+        TileRows tr0;
+        tile_rows(t, tr0);
         load_tile(tr0, kA, vA);
         compute(t, kA, vA);
       } else if (t + 64 == t_last) {  // two tiles: everything in flight at once, nothing extra
+        uint4 kA[4], vA[4], kB[4], vB[4];
+        TileRows tr, tr0;
+        tile_rows(t, tr0);
         tile_rows(t + 64, tr);
         load_tile(tr0, kA, vA);
         load_tile(tr, kB, vB);
@@ -385,8 +435,9 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
       } else if (!KLDS && t + 128 == t_last) {
         // three tiles (a sparse layer's usual share): a third set of registers keeps all of them in
         // flight behind one index round trip, instead of the third tile waiting for the first
-        uint4 kC[4], vC[4];
-        TileRows tr2;
+        uint4 kA[4], vA[4], kB[4], vB[4], kC[4], vC[4];
+        TileRows tr, tr0, tr2;
+        tile_rows(t, tr0);
         tile_rows(t + 64, tr);
         tile_rows(t + 128, tr2);
         load_tile(tr0, kA, vA);
@@ -396,6 +447,9 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
         compute(t + 64, kB, vB);
         compute(t + 128, kC, vC);
       } else {
+        uint4 kA[4], vA[4], kB[4], vB[4];
+        TileRows tr, tr0;
+        tile_rows(t, tr0);
         tile_rows(t + 64, tr);  // both lookups leave before the first one is awaited
         load_tile(tr0, kA, vA);
         while (true) {
@@ -505,9 +559,29 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
   }
 }
 
+// Kernel arguments are fetched by scalar loads that the compiler places next to their first use: a
+// chain of round trips through the scalar cache at the start of a pass that lasts a few microseconds.
+// Naming every field in an empty asm statement at the top makes all of them one batch of loads.
+template <typename X>
+__device__ __forceinline__ void fetch_now(const X& x) {
+  asm volatile("" ::"s"(x));
+}
+__device__ __forceinline__ void fetch_args_now(const RowList& r, const AttnWorkspace& w) {
+  fetch_now(r.k_base); fetch_now(r.v_base); fetch_now(r.token_stride); fetch_now(r.head_stride);
+  fetch_now(r.batch_stride); fetch_now(r.page_table); fetch_now(r.page_size); fetch_now(r.page_table_stride);
+  fetch_now(r.page_shift); fetch_now(r.page_stride); fetch_now(r.idx); fetch_now(r.idx_stride);
+  fetch_now(r.main_lens); fetch_now(r.max_main_len); fetch_now(r.tail_k); fetch_now(r.tail_v);
+  fetch_now(r.tail_token_stride); fetch_now(r.tail_head_stride); fetch_now(r.tail_batch_stride);
+  fetch_now(r.tail_lens); fetch_now(r.max_tail_len); fetch_now(r.score_lens); fetch_now(r.max_score_len);
+  fetch_now(w.part_o); fetch_now(w.part_lse); fetch_now(w.logits); fetch_now(w.max_splits);
+  fetch_now(w.split_rows); fetch_now(w.logits_stride); fetch_now(w.group_reduce); fetch_now(w.logit_heads);
+}
+
 template <typename T, int G, bool WITH_V, int MODE, bool LOGITS>
 __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q, RowList rows,
                                                         int hq, float scale, AttnWorkspace w) {
+  fetch_now(q);
+  fetch_args_now(rows, w);
   stage1_mfma_body<T, G, WITH_V, MODE, LOGITS, false>(q, rows, hq, scale, w, WindowFuse{});
 }
 
@@ -606,10 +680,7 @@ __global__ __launch_bounds__(1024) void score_raw_mfma(const T* __restrict__ q, 
     const int hcol = r16 < G ? r16 : G - 1;
     const T* qp = q + ((int64_t)(b * hq + g * G + hcol) * kD + 8 * j4);
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const uint4 v = *reinterpret_cast<const uint4*>(qp + 32 * s);
-      qf[s] = r16 < G ? v : make_uint4(0, 0, 0, 0);
-    }
+    for (int s = 0; s < 4; ++s) qf[s] = *reinterpret_cast<const uint4*>(qp + 32 * s);  // columns beyond G repeat head G-1
   }
   const T* kb = reinterpret_cast<const T*>(rows.k_base) + (int64_t)g * rows.head_stride + 8 * r16 +
                 (PAGED ? 0 : (int64_t)b * rows.batch_stride);
