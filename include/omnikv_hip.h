@@ -184,7 +184,7 @@ int okv_dense_attn_window(const void* q, const void* q_window, int64_t q_batch_s
  * seq_lens / k_per_seg: device int32[batch] or NULL (then max_seq_len / max_k
  * apply to every request).  idx_out rows beyond k_b are left untouched.
  * ws may be NULL: then one workgroup per request does all the work.  With a
- * workspace of okv_workspace_bytes(OKV_OP_TOPK) bytes, vectors of 16384 scores or
+ * workspace of okv_workspace_bytes(OKV_OP_TOPK) bytes, vectors of 14336 scores or
  * more are processed by many workgroups in chunked passes (the workspace needs no
  * preparation).
  */

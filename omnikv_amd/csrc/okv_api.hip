@@ -2,6 +2,8 @@
 #include <stdarg.h>
 #include <string.h>
 
+#include <algorithm>
+
 #include "okv_internal.h"
 
 namespace okv {
@@ -34,12 +36,30 @@ static int num_compute_units() {
   return cus;
 }
 
+// Local data share a workgroup may ask for on this device.
+int lds_bytes_per_workgroup() {
+  static int bytes = 0;
+  if (bytes == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) == hipSuccess && n > 0)
+      bytes = n;
+    else
+      bytes = 64 * 1024;
+  }
+  return bytes;
+}
+
 // Rows per split.  The pass is bandwidth-bound, so the grid is sized to what the chip holds at
 // once, every workgroup getting the same share of rows: all of them start together and finish
 // together, in one round when the split fits the row cap, else in the fewest equal rounds.
 // The attention kernels hold two workgroups per CU (their registers allow two waves per SIMD);
 // scoring alone could hold five and does best sized for three (measured at 128K: 50.6 us against
-// 53.1 sized for six).  The cap keeps the LDS staging of a scored split's logits small.
+// 53.1 sized for six).  A scored split stages its logits in LDS and hands them over in one burst
+// at its end, and every round of workgroups ends in such a burst, so the cap on its rows is what
+// the LDS of a CU lets the resident workgroups stage: 160 KB shared by two attention workgroups,
+// each with 16 KB of K staging and its logits (one row per q head of the group, or one per kv head
+// when the pass folds the group itself -- kind 3).
 static int choose_split_rows(int batch, int hq, int hkv, int total_rows, bool with_v,
                              bool with_logits, int kind) {
   const int forced = g_split_rows_override.load(std::memory_order_relaxed);
@@ -48,22 +68,37 @@ static int choose_split_rows(int batch, int hq, int hkv, int total_rows, bool wi
   // three and six per CU there (measured on 16 requests of 8K..32K tokens)
   // kind 2: the dense pass that carries a query window needs more than half a SIMD's registers per wave, so
   // one workgroup per CU is resident
-  const int64_t capacity = (int64_t)num_compute_units() * (kind == 2 ? 1 : batch <= 1 ? (with_v ? 2 : 3) : (with_v ? 3 : 6));
-  // a scored split stages G*rows fp32 logits in LDS: keep that within 33 KB (2112 rows at G = 4,
-  // what one round of a 128K context needs)
-  const int group = hkv > 0 && hq >= hkv ? hq / hkv : 1;
-  const int64_t cap_rows = with_logits ? (8448 / group) / 64 * 64 : kind == 2 ? 8192 : 4096;
+  const int group = kind == 3 ? 1 : hkv > 0 && hq >= hkv ? hq / hkv : 1;
   const int64_t work = (int64_t)(total_rows > 0 ? total_rows : 1) * hkv * (batch > 0 ? batch : 1);
-  for (int64_t rounds = 1;; ++rounds) {
-    int64_t rows = (work + rounds * capacity - 1) / (rounds * capacity);
-    rows = (rows + 63) / 64 * 64;
-    if (rounds == 1 && with_v && batch > 1 && rows <= 128) {
-      // a short pass is a chain of latencies: fewer, fatter workgroups
-      rows = (work + capacity * 2 / 3 - 1) / (capacity * 2 / 3);
+  // rows per split and rounds of workgroups for `per_cu` resident workgroups whose splits stage at
+  // most `logit_bytes` of logits
+  auto plan = [&](int per_cu, int64_t logit_bytes, int64_t* rounds_out) -> int {
+    const int64_t capacity = (int64_t)num_compute_units() * per_cu;
+    const int64_t cap_rows = with_logits ? std::min<int64_t>(logit_bytes / (4 * group) / 64 * 64, 8192) : kind == 2 ? 8192 : 4096;
+    for (int64_t rounds = 1;; ++rounds) {
+      int64_t rows = (work + rounds * capacity - 1) / (rounds * capacity);
       rows = (rows + 63) / 64 * 64;
+      if (rounds == 1 && with_v && batch > 1 && rows <= 128) {
+        // a short pass is a chain of latencies: fewer, fatter workgroups
+        rows = (work + capacity * 2 / 3 - 1) / (capacity * 2 / 3);
+        rows = (rows + 63) / 64 * 64;
+      }
+      if (rows <= cap_rows) {
+        *rounds_out = rounds;
+        return (int)rows;
+      }
     }
-    if (rows <= cap_rows) return (int)rows;
-  }
+  };
+  const int64_t three_share = 33 * 1024;  // logits three resident workgroups leave each other (next to their K staging)
+  const int64_t two_share = std::max<int64_t>(three_share, std::min<int64_t>(lds_bytes_per_workgroup(), 80 * 1024) - 17 * 1024);
+  int64_t rounds = 0;
+  if (kind == 2) return plan(1, three_share, &rounds);
+  if (batch > 1) return plan(with_v ? 3 : 6, three_share, &rounds);
+  if (with_v) return plan(2, two_share, &rounds);
+  // scoring alone: sized for three per CU unless two, with their longer splits, save a round of bursts
+  int64_t rounds2 = 0;
+  const int rows3 = plan(3, three_share, &rounds), rows2 = plan(2, two_share, &rounds2);
+  return with_logits && rounds2 < rounds ? rows2 : rows3;
 }
 
 size_t attn_workspace_bytes(int batch, int hq, int hkv, int d, int max_main, int max_tail,

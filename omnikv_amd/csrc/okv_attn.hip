@@ -242,6 +242,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void attn_merge(RowList rows, int hq, AttnWorkspace w,
                                                   T* __restrict__ out, int with_v,
                                                   int with_score_lse) {
+  fetch_now(out);
+  fetch_args_now(rows, w);
   merge_body<T>(rows, hq, w, out, with_v, with_score_lse, blockIdx.x, blockIdx.y);
 }
 
@@ -354,6 +356,9 @@ __global__ __launch_bounds__(256) void merge_and_finish(RowList rows, int hq, At
                                                         int head_reduce, int normalise,
                                                         float* __restrict__ scores,
                                                         int64_t score_stride) {
+  fetch_now(out);
+  fetch_now(scores);
+  fetch_args_now(rows, w);
   if ((int)blockIdx.x < merge_blocks)
     merge_body<T>(rows, hq, w, out, 1, 0, blockIdx.x, blockIdx.y);
   else
@@ -578,9 +583,12 @@ int okv_dense_attn(const void* q, const void* k_base, const void* v_base,
     score_lens = nullptr;
   }
   AttnWorkspace w;
+  // raw scores of 16-bit K are folded per kv head inside the pass: a quarter of the logits to stage, longer splits
+  const bool folds = scores && normalise == OKV_NORM_RAW && layout->dtype != OKV_F32 &&
+                     layout->num_q_heads > layout->num_kv_heads;
   rc = carve_attn_workspace(ws, ws_bytes, batch, layout->num_q_heads, layout->num_kv_heads,
                             layout->head_dim, max_seq_len, 0, max_score_len, true,
-                            scores != nullptr, &w);
+                            scores != nullptr, &w, folds ? 3 : 0);
   if (rc) return rc;
   RowList r;
   fill_main(&r, k_base, v_base, layout);

@@ -305,11 +305,12 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
   for (int e = 0; e < 8; ++e) acc[e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   const float sl2 = scale * kLog2e;
   const bool scored = LOGITS && begin < A;  // a scored split ends at or before A
-  float* slog = lds;  // [G][split_rows] scaled logits of the split; flushed before LDS is reused below
+  float* slog = lds;  // [G or 1][split_rows] scaled logits of the split; flushed before LDS is reused below
 
   // K staging of the streaming modes: 4 KB per wave behind everything else the block keeps in LDS
   int kst_off = stage1_lds_floats<G>(WITH_V);
-  if (LOGITS && G * w.split_rows > kst_off) kst_off = G * w.split_rows;
+  const int staged = (w.group_reduce ? 1 : G) * w.split_rows;  // one logits row per q head, or per kv head when folded
+  if (LOGITS && staged > kst_off) kst_off = staged;
   float* wlds = lds + kst_off;  // the window columns' states meet here at the end
   if (WINDOW) kst_off += kWindowLdsFloats;
   char* kstage = reinterpret_cast<char*>(lds + kst_off) + wave * 4096;
@@ -559,24 +560,6 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
   }
 }
 
-// Kernel arguments are fetched by scalar loads that the compiler places next to their first use: a
-// chain of round trips through the scalar cache at the start of a pass that lasts a few microseconds.
-// Naming every field in an empty asm statement at the top makes all of them one batch of loads.
-template <typename X>
-__device__ __forceinline__ void fetch_now(const X& x) {
-  asm volatile("" ::"s"(x));
-}
-__device__ __forceinline__ void fetch_args_now(const RowList& r, const AttnWorkspace& w) {
-  fetch_now(r.k_base); fetch_now(r.v_base); fetch_now(r.token_stride); fetch_now(r.head_stride);
-  fetch_now(r.batch_stride); fetch_now(r.page_table); fetch_now(r.page_size); fetch_now(r.page_table_stride);
-  fetch_now(r.page_shift); fetch_now(r.page_stride); fetch_now(r.idx); fetch_now(r.idx_stride);
-  fetch_now(r.main_lens); fetch_now(r.max_main_len); fetch_now(r.tail_k); fetch_now(r.tail_v);
-  fetch_now(r.tail_token_stride); fetch_now(r.tail_head_stride); fetch_now(r.tail_batch_stride);
-  fetch_now(r.tail_lens); fetch_now(r.max_tail_len); fetch_now(r.score_lens); fetch_now(r.max_score_len);
-  fetch_now(w.part_o); fetch_now(w.part_lse); fetch_now(w.logits); fetch_now(w.max_splits);
-  fetch_now(w.split_rows); fetch_now(w.logits_stride); fetch_now(w.group_reduce); fetch_now(w.logit_heads);
-}
-
 template <typename T, int G, bool WITH_V, int MODE, bool LOGITS>
 __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q, RowList rows,
                                                         int hq, float scale, AttnWorkspace w) {
@@ -585,8 +568,9 @@ __global__ __launch_bounds__(256) void attn_stage1_mfma(const T* __restrict__ q,
   stage1_mfma_body<T, G, WITH_V, MODE, LOGITS, false>(q, rows, hq, scale, w, WindowFuse{});
 }
 
-// The dense pass with the window columns: capped at the registers that let two workgroups share a
-// CU, like the pass without them.
+// The dense pass with the window columns.  The 64 registers of window query fragments put a wave
+// beyond half a SIMD's register file, so one workgroup is resident per CU and the splits are sized
+// for that (capping the registers for two per CU spills and is slower).
 template <typename T, int G>
 __global__ __launch_bounds__(256) void attn_stage1_window_mfma(const T* __restrict__ q, RowList rows,
                                                                   int hq, float scale, AttnWorkspace w,
@@ -601,7 +585,8 @@ static void launch_one(const void* q, const RowList& rows, int hq, int hkv, int 
   if constexpr (WINDOW) kern_ptr = reinterpret_cast<const void*>(attn_stage1_window_mfma<T, G>);
   else kern_ptr = reinterpret_cast<const void*>(attn_stage1_mfma<T, G, WITH_V, MODE, LOGITS>);
   size_t lds_floats = stage1_lds_floats<G>(WITH_V);  // the logits staging aliases the merge buffers
-  if (LOGITS && (size_t)G * w.split_rows > lds_floats) lds_floats = (size_t)G * w.split_rows;
+  const size_t staged = (size_t)(w.group_reduce ? 1 : G) * w.split_rows;
+  if (LOGITS && staged > lds_floats) lds_floats = staged;
   if (WINDOW) lds_floats += kWindowLdsFloats;
   if (stage1_k_through_lds(MODE)) lds_floats += 4 * 1024;  // 4 KB of K staging per wave
   const size_t lds_bytes = lds_floats * sizeof(float);
@@ -853,8 +838,11 @@ bool launch_stage1_mfma(int dtype, const void* q, const RowList& rows, int hq, i
                         hipStream_t stream) {
   // token strides are used as 32-bit multipliers
   if (rows.token_stride >= (1ll << 31) || rows.tail_token_stride >= (1ll << 31)) return false;
-  // the split's logits are staged in LDS next to the merge buffers
-  if (write_logits && (size_t)(hq / hkv) * w.split_rows * sizeof(float) > 48 * 1024) return false;
+  // the split's logits (one row per q head of the group, or one per kv head when the pass folds the
+  // group) are staged in LDS next to the K staging
+  const size_t logit_rows = w.group_reduce ? 1 : hq / hkv;
+  if (write_logits && logit_rows * w.split_rows * sizeof(float) + 20 * 1024 > (size_t)lds_bytes_per_workgroup())
+    return false;
   if (dtype == OKV_BF16)
     return launch_t<BF16>(q, rows, hq, hkv, batch, scale, w, with_v, write_logits, stream);
   if (dtype == OKV_F16)

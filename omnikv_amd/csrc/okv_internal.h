@@ -143,6 +143,24 @@ struct AttnWorkspace {
   int32_t logit_heads;   // rows of `logits` per request: Hq, or Hkv when group_reduce
 };
 
+// Kernel arguments are fetched by scalar loads that the compiler places next to their first use: a
+// chain of round trips through the scalar cache at the start of a pass that lasts a few microseconds.
+// Naming every field in an empty asm statement at the top makes all of them one batch of loads.
+template <typename X>
+__device__ __forceinline__ void fetch_now(const X& x) {
+  asm volatile("" ::"s"(x));
+}
+__device__ __forceinline__ void fetch_args_now(const RowList& r, const AttnWorkspace& w) {
+  fetch_now(r.k_base); fetch_now(r.v_base); fetch_now(r.token_stride); fetch_now(r.head_stride);
+  fetch_now(r.batch_stride); fetch_now(r.page_table); fetch_now(r.page_size); fetch_now(r.page_table_stride);
+  fetch_now(r.page_shift); fetch_now(r.page_stride); fetch_now(r.idx); fetch_now(r.idx_stride);
+  fetch_now(r.main_lens); fetch_now(r.max_main_len); fetch_now(r.tail_k); fetch_now(r.tail_v);
+  fetch_now(r.tail_token_stride); fetch_now(r.tail_head_stride); fetch_now(r.tail_batch_stride);
+  fetch_now(r.tail_lens); fetch_now(r.max_tail_len); fetch_now(r.score_lens); fetch_now(r.max_score_len);
+  fetch_now(w.part_o); fetch_now(w.part_lse); fetch_now(w.logits); fetch_now(w.max_splits);
+  fetch_now(w.split_rows); fetch_now(w.logits_stride); fetch_now(w.group_reduce); fetch_now(w.logit_heads);
+}
+
 // The last W query positions of every q head riding along a dense pass (window selectors): the
 // pass then also leaves, per scored split, the log-sum-exp of every (position, head) column's
 // logits, which is what the first of the window selector's two passes over K computes.
@@ -156,7 +174,9 @@ struct WindowFuse {
 
 size_t attn_workspace_bytes(int batch, int hq, int hkv, int d, int max_main, int max_tail,
                             int max_score, bool with_v, bool with_logits,
-                            int* split_rows, int* max_splits, int kind = 0);  // kind: 0 plain, 1 gather, 2 with a query window
+                            int* split_rows, int* max_splits,
+                            int kind = 0);  // kind: 0 plain, 1 gather, 2 with a query window, 3 logits folded per kv head
+int lds_bytes_per_workgroup();
 int carve_attn_workspace(void* ws, size_t ws_bytes, int batch, int hq, int hkv, int d,
                          int max_main, int max_tail, int max_score, bool with_v,
                          bool with_logits, AttnWorkspace* out, int kind = 0);
