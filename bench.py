@@ -384,6 +384,8 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
 
+    from omnikv_amd import _lib as okv_lib
+    okv_lib.use_diag_build()  # the product's kernels + the measurement hooks (split pass alone, load-only floor)
     from omnikv_amd import ops
     from omnikv_amd._lib import check, lib
 

@@ -11,6 +11,7 @@ import os
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "libomnikv_hip.so")
+DIAG_LIB_PATH = os.path.join(_PKG, "libomnikv_hip_diag.so")  # measurement build: + the okv_diag_* hooks
 
 OKV_F32, OKV_BF16, OKV_F16 = 0, 1, 2
 OKV_REDUCE_MAX, OKV_REDUCE_SUM = 0, 1
@@ -91,14 +92,15 @@ def _declare(l):
     l.okv_workspace_bytes.argtypes = [C.c_int, C.POINTER(Shape), C.POINTER(sz)]
     l.okv_set_option.restype = C.c_int
     l.okv_set_option.argtypes = [C.c_char_p, C.c_int]
-    l.okv_diag_split_pass_only.restype = C.c_int  # measurement hook, not part of the public header
-    l.okv_diag_split_pass_only.argtypes = [C.c_int]
-    l.okv_diag_split_geometry.restype = C.c_int
-    l.okv_diag_split_geometry.argtypes = [C.c_int, C.POINTER(Shape), C.POINTER(i32), C.POINTER(i32)]
-    l.okv_diag_gather_floor.restype = C.c_int
-    l.okv_diag_gather_floor.argtypes = [vp, vp, C.POINTER(KVLayout), vp, i32, i32, i32, vp, vp]
-    l.okv_diag_empty_launch.restype = C.c_int
-    l.okv_diag_empty_launch.argtypes = [vp, vp]
+    if hasattr(l, "okv_diag_split_pass_only"):  # the measurement build only; not part of the public header
+        l.okv_diag_split_pass_only.restype = C.c_int
+        l.okv_diag_split_pass_only.argtypes = [C.c_int]
+        l.okv_diag_split_geometry.restype = C.c_int
+        l.okv_diag_split_geometry.argtypes = [C.c_int, C.POINTER(Shape), C.POINTER(i32), C.POINTER(i32)]
+        l.okv_diag_gather_floor.restype = C.c_int
+        l.okv_diag_gather_floor.argtypes = [vp, vp, C.POINTER(KVLayout), vp, i32, i32, i32, vp, vp]
+        l.okv_diag_empty_launch.restype = C.c_int
+        l.okv_diag_empty_launch.argtypes = [vp, vp]
     l.okv_score.restype = C.c_int
     l.okv_score.argtypes = [vp, vp, C.POINTER(KVLayout), vp, i32, i32, i32, i32, f32, vp, i64, vp, sz, vp]
     l.okv_score_window.restype = C.c_int
@@ -138,16 +140,29 @@ def _declare(l):
     l.okv_offload_stage.argtypes = [vp, i64, vp, i32, vp, i32, vp, vp, vp]
 
 
+_want_diag = False
+
+
+def use_diag_build() -> None:
+    """Benchmarks call this before anything else touches the library: the process then loads the
+    measurement build (the product's sources + the okv_diag_* hooks) instead of the product library."""
+    global _want_diag
+    if _lib is not None and not hasattr(_lib, "okv_diag_split_pass_only"):
+        raise OmniKVLibraryError("the product library is already loaded: call use_diag_build() first")
+    _want_diag = True
+
+
 def lib():
     """The loaded library; raises if it has not been built."""
     global _lib
     if _lib is None:
-        if not os.path.exists(LIB_PATH):
+        path = DIAG_LIB_PATH if _want_diag else LIB_PATH
+        if not os.path.exists(path):
             raise OmniKVLibraryError(
-                f"{LIB_PATH} is missing: build it with `python omnikv_amd/csrc/build.py` "
+                f"{path} is missing: build it with `python omnikv_amd/csrc/build.py` "
                 "(hipcc, gfx950). There is no fallback path."
             )
-        l = C.CDLL(LIB_PATH)
+        l = C.CDLL(path)
         _declare(l)
         _lib = l
     return _lib

@@ -29,7 +29,8 @@ import torch
 from . import ops
 from ._lib import check, lib
 
-__all__ = ["OmniKVMultiStageCache", "WOPackCache", "get_cache_cls", "get_idx_iou_score", "layer_schedule"]
+__all__ = ["OmniKVMultiStageCache", "WOPackCache", "OmniKVLazyCache", "get_cache_cls", "get_idx_iou_score",
+           "layer_schedule"]
 
 
 def layer_schedule(full_attn_layers, num_hidden_layers: int, num_wait_load_layers: int):
@@ -271,6 +272,14 @@ class OmniKVMultiStageCache:
                 self._host_kv[layer_idx] = host
             elif host.shape[0] != n:
                 raise NotImplementedError("an offloaded layer takes its prompt in one prefill call")
+            else:
+                # the same pinned rows are about to hold another prompt: whatever was staged from them,
+                # and the incremental mode's record of which tokens sit in which slots, is stale
+                self._plan.pop(self.layer_state[layer_idx][1], None)
+                self._staged_for.pop(layer_idx, None)
+                self._part_src.pop(layer_idx, None)
+                self.part_key.pop(layer_idx, None)
+                self.part_value.pop(layer_idx, None)
             if not key_states.is_cuda:  # rows that already live on the host (an adopted cache)
                 host[:, 0].copy_(key_states[0].permute(1, 0, 2))
                 host[:, 1].copy_(value_states[0].permute(1, 0, 2))
@@ -732,10 +741,33 @@ def get_idx_iou_score(new_idx: torch.Tensor, old_idx: torch.Tensor) -> float:
     return inter / new_idx.shape[0]
 
 
+class OmniKVLazyCache(OmniKVMultiStageCache):
+    """`cache_cls: lazy` (modeling/spec_cache.py:523-557): the multi-stage cache that keeps the rows it has
+    staged when a new selection overlaps the one in use by more than `skip_threshold` of its indices
+    (OmniKVLazyCache.set_out_idx; the reference's default threshold is 0.4 of `get_idx_iou_score`).  The
+    reference pairs it with a model class of its own that feeds it one selection per step; here it is the
+    `multi` cache with that threshold switched on, behind the same interface."""
+
+    DEFAULT_SKIP_THRESHOLD = 0.4
+
+    def __init__(self, full_attn_layers: List, num_hidden_layers, num_wait_load_layers=2, real_offload=True,
+                 **kwargs):
+        if kwargs.get("skip_threshold") is None:
+            kwargs["skip_threshold"] = self.DEFAULT_SKIP_THRESHOLD
+        super().__init__(full_attn_layers, num_hidden_layers, num_wait_load_layers, real_offload, **kwargs)
+
+    @staticmethod
+    def from_dynamic_cache(cache, full_attn_layers: List, num_hidden_layers, num_wait_load_layers=2,
+                           real_offload=True, **kwargs):
+        return OmniKVMultiStageCache.from_dynamic_cache(cache, full_attn_layers, num_hidden_layers,
+                                                        num_wait_load_layers, real_offload, _cls=OmniKVLazyCache, **kwargs)
+
+
 def get_cache_cls(config):
-    """modeling/spec_cache.py:829-837, restricted to the classes this build provides."""
-    name2cls = {"multi": OmniKVMultiStageCache, "without_pack": WOPackCache}
+    """modeling/spec_cache.py:829-837.  `lazy` is the multi-stage cache with re-selection skipping on;
+    `default` (the baseline without selection) and `eff` (broken upstream) belong to other model paths."""
+    name2cls = {"multi": OmniKVMultiStageCache, "without_pack": WOPackCache, "lazy": OmniKVLazyCache}
     name = config.get("cache_cls", "default")
     if name not in name2cls:
-        raise NotImplementedError(f"cache_cls={name!r}: 'multi' and 'without_pack' are built here")
+        raise NotImplementedError(f"cache_cls={name!r}: 'multi', 'without_pack' and 'lazy' are built here")
     return name2cls[name]

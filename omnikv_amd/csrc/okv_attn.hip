@@ -368,7 +368,9 @@ __global__ __launch_bounds__(256) void merge_and_finish(RowList rows, int hq, At
 
 // ----------------------------------------------------------------- launch
 std::atomic<int> g_attn_variant{0};  // 0 = pick per dtype, 1 = portable VALU stage 1 everywhere
-std::atomic<int> g_split_pass_only{0};  // diagnostic (okv_diag_split_pass_only): no merge / finish launch
+#ifdef OKV_DIAG
+std::atomic<int> g_split_pass_only{0};  // measurement build only (okv_diag_split_pass_only): no merge / finish launch
+#endif
 
 bool launch_stage1_mfma(int dtype, const void* q, const RowList& rows, int hq, int hkv, int batch,
                         float scale, const AttnWorkspace& w, bool with_v, bool write_logits,
@@ -425,9 +427,10 @@ static int launch_typed(const void* q, const RowList& rows, const okv_kv_layout_
   const int ftok = finish_tokens_for(w.split_rows, rows.max_score_len);
   const int finish_blocks = want_scores ? (rows.max_score_len + ftok - 1) / ftok : 0;
   const AttnWorkspace& uw = *used;
-  if (g_split_pass_only.load(std::memory_order_relaxed)) {
-    // measurement hook: the split pass alone
-  } else if (finish_blocks > 0 && hq <= kMaxFinishHeads) {
+#ifdef OKV_DIAG
+  if (g_split_pass_only.load(std::memory_order_relaxed)) return OKV_OK;  // measurement hook: the split pass alone
+#endif
+  if (finish_blocks > 0 && hq <= kMaxFinishHeads) {
     // one launch: the merge of the outputs next to the finishing of the scores
     const dim3 grid((with_v ? hq : 0) + finish_blocks, batch);
     if (ftok == 512)
@@ -525,13 +528,16 @@ int okv_set_option(const char* name, int value) {
   return OKV_ERR_INVALID;
 }
 
-// Measurement hook, deliberately absent from the public header: with 1 the attention / scoring
-// entry points launch their split pass alone (outputs are then not produced), so that a timer
-// around the call measures that kernel.  Process-wide; never set it in a serving process.
+#ifdef OKV_DIAG
+// Measurement hook of the measurement build (compiled with -DOKV_DIAG into libomnikv_hip_diag.so; the
+// product library does not contain it): with 1 the attention / scoring entry points launch their
+// split pass alone (outputs are then not produced), so that a timer around the call measures that
+// kernel.  Process-wide.
 int okv_diag_split_pass_only(int on) {
   g_split_pass_only.store(on ? 1 : 0, std::memory_order_relaxed);
   return OKV_OK;
 }
+#endif
 
 int okv_score(const void* q, const void* k_base, const okv_kv_layout_t* layout,
               const int32_t* score_lens, int32_t max_score_len, int32_t batch,

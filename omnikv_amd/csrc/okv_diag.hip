@@ -1,6 +1,7 @@
-// Measurement hooks of libomnikv_hip.so.  Nothing here is on the product path and nothing here
-// is declared in the public header: these entry points exist so that the benchmark can put an
-// attainable bound next to a kernel's time, measured on the same device in the same run.
+// Measurement hooks.  This file is part of the measurement build only (libomnikv_hip_diag.so, which
+// bench.py and the microbenchmark load); the product library libomnikv_hip.so is built without it.
+// Nothing here is declared in the public header: these entry points exist so that the benchmark can
+// put an attainable bound next to a kernel's time, measured on the same device in the same run.
 #include "okv_device.h"
 #include "okv_internal.h"
 

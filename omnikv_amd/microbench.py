@@ -53,6 +53,8 @@ def main():
     ap.add_argument("--attn-variant", type=int, default=0)
     args = ap.parse_args()
 
+    from . import _lib as okv_lib
+    okv_lib.use_diag_build()  # the product's kernels + the measurement hooks
     check(lib().okv_set_option(b"split_rows", args.split_rows))
     check(lib().okv_set_option(b"attn_variant", args.attn_variant))
     dev = torch.device("cuda:0")

@@ -435,6 +435,16 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: Optiona
     return out if residual is None else (out, total)
 
 
+def _check_rope_tables(cos: torch.Tensor, sin: torch.Tensor, bsz: int, d: int) -> None:
+    """The kernels read one row of d cos / sin values per request, back to back: a broadcast (1, 1, d) table
+    next to bsz > 1 would be read past its end."""
+    if d != 128:
+        raise ValueError("the rotary kernels are built for head_dim 128")
+    if tuple(cos.shape) != (bsz, 1, d) or tuple(sin.shape) != (bsz, 1, d):
+        raise ValueError(f"cos / sin must be (bsz, 1, head_dim) = ({bsz}, 1, {d}), one row per request; "
+                         f"got {tuple(cos.shape)} and {tuple(sin.shape)} (expand a shared row first)")
+
+
 def rope(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, num_q_heads: int,
          num_kv_heads: int) -> Tuple[torch.Tensor, torch.Tensor]:
     """Rotary embedding of one position per request: q (bsz, 1, Hq*D) and k (bsz, 1, Hkv*D) as the
@@ -444,6 +454,7 @@ def rope(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
     d = cos.shape[-1]
     if q.shape[1] != 1 or q.shape[-1] != num_q_heads * d or k.shape[-1] != num_kv_heads * d:
         raise ValueError("q / k must be (bsz, 1, heads * head_dim)")
+    _check_rope_tables(cos, sin, bsz, d)
     q_out = torch.empty((bsz, num_q_heads, 1, d), dtype=q.dtype, device=q.device)
     k_out = torch.empty((bsz, num_kv_heads, 1, d), dtype=q.dtype, device=q.device)
     check(lib().okv_rope(q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), cos.data_ptr(), sin.data_ptr(), bsz,
@@ -456,9 +467,12 @@ def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Te
                 pos) -> torch.Tensor:
     """`rope` whose rotated k row and the v row are written into k_store / v_store (bsz, Hkv, capacity, D) at
     token position `pos` (an int, or a one-element int64 GPU tensor read by the kernel); returns the rotated
-    q (bsz, Hq, 1, D).  okv_rope_append."""
+    q (bsz, Hq, 1, D).  Every request of the batch is written at the SAME position (the static decode
+    path advances all requests together); nothing on the device checks a device position against the
+    store's capacity -- the cache's host-side step count does.  okv_rope_append."""
     dt = _same(q, k, v, cos, sin)
     bsz, d = q.shape[0], cos.shape[-1]
+    _check_rope_tables(cos, sin, bsz, d)
     if k_store.dtype != q.dtype or k_store.stride() != v_store.stride() or k_store.stride(-1) != 1:
         raise ValueError("k_store / v_store must share dtype with q and strides with each other")
     if k_store.shape[0] != bsz or k_store.shape[1] != num_kv_heads or k_store.shape[3] != d:

@@ -143,6 +143,37 @@ def score_tokens_by_kv_head(
     raise NotImplementedError(selector_cls)
 
 
+def score_window_by_kv_head(
+    q: torch.Tensor, k: torch.Tensor, consider_len: int, selector_cls: str = "uniform"
+) -> torch.Tensor:
+    """`score_tokens` of the window selectors (`uniform`, `exp`; modeling/omnikv.py:59-105)
+    evaluated one kv head at a time for the long contexts: per window position the softmax is
+    per q head and the head reduction a max, so the max over all q heads is the max over kv
+    heads of the max over each group; the positions are then added up in the reference's
+    order (`attn_sum + s`, or `attn_sum * 2**-1 + s` for `exp`).  Holds (group, W, N) logits of
+    one kv head at a time instead of the (Hq, N) of every position over a 4x repeated K."""
+    if selector_cls not in ("uniform", "exp"):
+        raise NotImplementedError(selector_cls)
+    hq, hkv = q.shape[1], k.shape[1]
+    g = hq // hkv
+    k = k[:, :, :consider_len]
+    per_pos = None  # (b, W, N): max over the q heads seen so far of their softmax probabilities
+    for i in range(hkv):
+        p = torch.nn.functional.softmax(attn_logits(q[:, g * i: g * (i + 1)], k[:, i: i + 1]), dim=-1)
+        p = torch.max(p, dim=1).values
+        per_pos = p if per_pos is None else torch.maximum(per_pos, p)
+    attn_sum = None
+    for w in range(per_pos.shape[1]):
+        s = per_pos[:, w]
+        if attn_sum is None:
+            attn_sum = s
+        elif selector_cls == "uniform":
+            attn_sum = attn_sum + s
+        else:
+            attn_sum = attn_sum * (2.0 ** -1) + s
+    return attn_sum
+
+
 # --------------------------------------------------------------------------
 # top-k (modeling/omnikv.py:47-48,109-110)
 # --------------------------------------------------------------------------

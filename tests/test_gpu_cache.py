@@ -264,6 +264,43 @@ def test_incremental_staging_fetches_only_rows_that_are_new(overlap):
         assert torch.equal(dk.cpu(), rk) and torch.equal(dv.cpu(), rv), i
 
 
+def test_second_prompt_of_the_same_length_invalidates_what_incremental_staging_remembers():
+    """The pinned rows of an offloaded layer are rewritten in place by a second prefill of the same
+    length.  The slot maps of the incremental mode then describe rows of the OLD prompt: a selection that
+    repeats tokens of the previous one must fetch them again, not reuse the stale staged rows."""
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(77)
+    n, kk, L, hq, hkv, d = 1200, 120, 4, 32, 8, 128
+    full = orc.full_attn_layers_from_select_layers([0], L)  # filter 0, wait 1, sparse 2..3
+    dut = OmniKVMultiStageCache(full, L, 1, True, max_new_tokens=8, offload_mode="incremental")
+    idx = torch.randperm(n, generator=g)[:kk].sort().values
+    for prompt in range(2):
+        dut.stage = "prefill"
+        keys = [torch.randn((1, hkv, n, d), generator=g).to(dtype) for _ in range(L)]
+        vals = [torch.randn((1, hkv, n, d), generator=g).to(dtype) for _ in range(L)]
+        if prompt == 1:  # a fresh prompt in the same cache object: dense stores start over
+            for st in dut._store.values():
+                st.len = 0
+            dut._tail.clear()
+            dut.tail_k.clear()
+            dut.tail_v.clear()
+        for i in range(L):
+            dut.update(keys[i].to(DEV), vals[i].to(DEV), i)
+        dut.stage = "decoding"
+        dut.set_idx_on_gpu(idx[None].to(DEV), 0)  # the SAME tokens both times
+        assert dut.last_fetch_count(0) == kk, prompt  # nothing of the first prompt's staging is reused
+        for i in (2, 3):
+            q = torch.randn((1, hq, 1, d), generator=g).to(dtype)
+            k1 = torch.randn((1, hkv, 1, d), generator=g).to(dtype)
+            v1 = torch.randn((1, hkv, 1, d), generator=g).to(dtype)
+            dut.append(k1.to(DEV), v1.to(DEV), i)
+            pk = torch.cat([orc.gather_rows(keys[i], idx), k1], dim=-2)
+            pv = torch.cat([orc.gather_rows(vals[i], idx), v1], dim=-2)
+            want = orc.gqa_attention(q.float(), pk.float(), pv.float())[:, :, 0]
+            out = dut.attend(q.to(DEV), i).cpu().float()
+            assert (out - want).abs().max() < TOL[dtype], (prompt, i)
+
+
 def test_incremental_staging_is_refused_where_layers_stage_themselves():
     from omnikv_amd.cache import WOPackCache
     with pytest.raises(ValueError, match="incremental"):
@@ -291,6 +328,16 @@ def test_lazy_reselection_skips_similar_selections():
     assert dut.num_skipped_selections == 1 and torch.equal(dut._idx[0].cpu(), a.cpu().to(torch.int32))
     dut.set_idx_on_gpu(c, 0)
     assert dut.num_skipped_selections == 1 and torch.equal(dut._idx[0].cpu(), c.cpu().to(torch.int32))
+    # cache_cls: lazy is that cache with the reference's threshold of 0.4: b (2/3 shared) is skipped, c (1/3) taken
+    from omnikv_amd.cache import get_cache_cls
+    from omnikv_amd.config import OmniKVConfig
+    lazy = get_cache_cls(OmniKVConfig(cache_cls="lazy"))(full, L, 1, False, max_new_tokens=8)
+    for i in range(L):
+        lazy.update(torch.randn((1, 8, n, 128), generator=g).to(DEV), torch.randn((1, 8, n, 128), generator=g).to(DEV), i)
+    lazy.stage = "decoding"
+    for sel in (a, b, c):
+        lazy.set_idx_on_gpu(sel, 0)
+    assert lazy.num_skipped_selections == 1 and torch.equal(lazy._idx[0].cpu(), c.cpu().to(torch.int32))
     # default: every selection is taken, as the reference's multi-stage cache does
     ref = OmniKVMultiStageCache(full, L, 1, False)
     ref.set_idx_on_gpu(a, 0)

@@ -2,6 +2,9 @@
 (batch 1, bf16, the sink + heavy-hitter key distribution) and the batch of 16 ragged
 requests of 8192..32768 tokens on a paged pool with 16-token pages.
 
+Selectors: `last`, `softmax_before_last` (the reference's default, omnikv.py:139), the benchmark's
+`softmax_sum_last`, and the window selectors `uniform` / `exp` with 16 positions.
+
 Bars: scores within 1e-4 of the oracle's relative to the row's largest magnitude; top-k
 bit-exact on identical fp32 scores; on the kernel's own scores every index that differs from
 the oracle's selection is a provable near-tie (parity_helpers.assert_near_tie_only); attention within
@@ -43,7 +46,7 @@ def test_filter_layer_op_matches_oracle_at_benchmark_size(n, ks):
     assert (got_dense[0].cpu().float() - want_dense).abs().max() < ATTN_TOL
 
     qn = synth.fresh_q().to(DT)
-    for sel in ("last", "softmax_sum_last"):
+    for sel in ("last", "softmax_before_last", "softmax_sum_last"):
         want = (orc.score_tokens_by_kv_head if by_head else orc.score_tokens)(qf, kf, n, sel)
         alone = ops.score(qd, kd[:, :, :n], selector=sel)
         out, fused = ops.dense_attn(qd, kd, vd, selector=sel, score_len=n)
@@ -52,7 +55,7 @@ def test_filter_layer_op_matches_oracle_at_benchmark_size(n, ks):
         assert _rel(fused.cpu(), want) < SCORE_TOL, sel
         # the fused pass also is the layer's attention, over all n + 1 rows
         assert (out[0].cpu().float() - want_dense).abs().max() < ATTN_TOL
-        if "softmax" in sel:
+        if sel == "softmax_sum_last":
             assert abs(float(fused.double().sum()) - HQ) < 1e-2
         for kk in ks:
             want_idx = orc.select_topk_stable(want, kk)
@@ -78,6 +81,43 @@ def test_filter_layer_op_matches_oracle_at_benchmark_size(n, ks):
             assert (got_sp[0].cpu().float() - want_sp).abs().max() < ATTN_TOL, (sel, kk)
             # the materialised gather is a pure copy of the oracle's rows
             assert torch.equal(ops.gather_rows(kd[:, :, :n], idx).cpu(), orc.gather_rows(k, want_idx[0]))
+
+
+@pytest.mark.parametrize("n", [131072, 450000])
+def test_window_selectors_match_oracle_at_benchmark_size(n):
+    """`uniform` and `exp` (modeling/omnikv.py:59-105) with a window of 16 positions at the benchmark's
+    context lengths, through okv_score_window and through the filter layer's two-pass form
+    okv_dense_attn_window, against the oracle evaluated one kv head at a time.  450000 rows are where the
+    window passes take their largest split count."""
+    w = 16
+    q1, k, v = synth.filter_layer_inputs(n)
+    g = torch.Generator().manual_seed(n + 5)
+    # the window: the benchmark's query as the newest position, fifteen older ones scattered around it
+    qw = torch.cat([q1 + 0.5 * torch.randn((1, HQ, w - 1, D), generator=g), q1], dim=2).to(DT)
+    k, v = k.to(DT), v.to(DT)
+    tk, tv = torch.randn((1, HKV, 1, D), generator=g).to(DT), torch.randn((1, HKV, 1, D), generator=g).to(DT)
+    kd = torch.cat([k, tk], dim=2).to(DEV)
+    vd = torch.cat([v, tv], dim=2).to(DEV)
+    qd = qw.to(DEV)
+    assert ops.window_supported(qd, kd)
+    q_last = qd[:, :, -1:].contiguous()
+    want_dense = orc.gqa_attention_by_kv_head(qw[:, :, -1:].float(), torch.cat([k, tk], 2).float(),
+                                              torch.cat([v, tv], 2).float())[0, :, 0]
+    kk = int(0.067 * n)
+    for sel in ("uniform", "exp"):
+        want = orc.score_window_by_kv_head(qw.float(), k.float(), n, sel)
+        alone = ops.score_window(qd, kd[:, :, :n], score_len=n, selector=sel)
+        out, fused = ops.dense_attn_window(q_last, qd, kd, vd, selector=sel, score_len=n)
+        assert alone.shape == fused.shape == want.shape == (1, n)
+        assert _rel(alone.cpu(), want) < SCORE_TOL, sel
+        assert _rel(fused.cpu(), want) < SCORE_TOL, sel
+        assert (out[0].cpu().float() - want_dense).abs().max() < ATTN_TOL, sel
+        want_idx = orc.select_topk_stable(want, kk)
+        assert torch.equal(ops.topk(want.to(DEV), kk).cpu().to(torch.int64), want_idx), sel
+        for got in (alone, fused):
+            own = ops.topk(got, kk).cpu()[0].to(torch.int64)
+            assert torch.all(own[1:] > own[:-1])
+            assert_near_tie_only(got[0].cpu(), want[0], own, want_idx[0], kk)
 
 
 def test_batch16_ragged_paged_matches_oracle_at_benchmark_size():

@@ -119,9 +119,63 @@ def test_greedy_decode_matches_oracle(selector_cls, real_offload):
         if float(top2[0] - top2[1]) > 1e-2:
             assert int(got[0, 0].argmax()) == int(want[0, 0].argmax())
             agree += 1
+    assert agree >= steps - 1  # at most one step's top two logits were too close to call
     assert cache.get_seq_length() == n + steps
     if real_offload:
         cache._join_worker()
+
+
+class _CallCounter:
+    """Wraps a function of the ops module and counts its calls."""
+
+    def __init__(self, monkeypatch, name):
+        from omnikv_amd import ops
+        self.calls = 0
+        inner = getattr(ops, name)
+
+        def wrapped(*a, **kw):
+            self.calls += 1
+            return inner(*a, **kw)
+
+        monkeypatch.setattr(ops, name, wrapped)
+
+
+@pytest.mark.parametrize("selector_cls", ["uniform", "exp"])
+@pytest.mark.parametrize("real_offload", [False, True])
+def test_greedy_decode_bf16_window_selectors_take_the_fused_filter_layer(selector_cls, real_offload, monkeypatch):
+    """The 16-bit model path of the window selectors: the filter layer's attention and its first scoring
+    pass are one call (okv_dense_attn_window), through the steps in which the window still overlaps the
+    prompt (forced positions appended) and beyond.  Reference: the oracle runner in fp32 on the same
+    bf16-rounded weights, teacher-forced.  bf16 activations round differently from fp32 ones, so logits are
+    compared within 3% of their range and tokens wherever the oracle's top two are further apart than that."""
+    torch.manual_seed(0)
+    cfg = _config(selector_cls, real_offload)
+    lm = OmniKVMulLM(SHAPE, cfg).float()
+    lm.init_weights(seed=3, std=0.08)
+    lm = lm.to(torch.bfloat16)
+    ref = _OracleRunner(copy.deepcopy(lm).float(), _config(selector_cls, real_offload))
+    dut = lm.to(DEV)
+    fused = _CallCounter(monkeypatch, "dense_attn_window")
+    n, steps = 500, 7  # window_size 4: steps 1..3 append forced prompt positions, 4.. do not
+    ids = torch.randint(0, SHAPE.vocab_size, (1, n), generator=torch.Generator().manual_seed(1))
+    want = ref.forward(ids)
+    got, cache = dut.forward(ids.to(DEV), None, max_new_tokens=16)
+    scale = float(want.abs().max())
+    assert (got.cpu() - want).abs().max() < 0.03 * scale
+    agree = checked = 0
+    for t in range(steps):
+        tok = want[:, -1].argmax(-1, keepdim=True)
+        want = ref.forward(tok)
+        got, cache = dut.forward(tok.to(DEV), cache)
+        assert (got.cpu() - want).abs().max() < 0.03 * scale, (selector_cls, real_offload, t)
+        top2 = want[0, 0].topk(2).values
+        if float(top2[0] - top2[1]) > 0.06 * scale:
+            checked += 1
+            agree += int(got[0, 0].argmax()) == int(want[0, 0].argmax())
+    assert agree == checked
+    assert fused.calls == 2 * steps  # both filter layers, every decode step
+    sel = cache._idx[1]
+    assert sel.dtype == torch.int32 and sel.shape[1] == int(0.1 * n)  # forced window gone: k rows again
 
 
 def test_generate_greedy_and_error_paths():
@@ -140,6 +194,57 @@ def test_generate_greedy_and_error_paths():
     _, cache = lm2.forward(ids, None)
     with pytest.raises(ValueError):  # modeling/omnikv.py:213-214
         lm2.forward(ids[:, :1], cache)
+
+
+@pytest.mark.parametrize("selector_cls,offload", [("uniform", True), ("exp", "incremental"), ("uniform", False)])
+def test_graph_replayed_bf16_window_decode_takes_the_fused_branch(selector_cls, offload, monkeypatch):
+    """Static decode of a 16-bit model with a window selector, eager static steps and graph replays, with
+    and without the host tier: the captured step holds okv_dense_attn_window (the fused filter layer writing
+    into the fixed index buffer, the copy stream staging behind it), and every replay reproduces what the
+    same number of eager STATIC steps of a second, identically initialised model produce -- the same
+    kernels on the same shapes, so bit for bit."""
+    ids = torch.randint(0, SHAPE.vocab_size, (1, 400), generator=torch.Generator().manual_seed(4)).to(DEV)
+    kw = {"offload_mode": offload} if isinstance(offload, str) else {}
+    steps = 6
+
+    def fresh():
+        lm = OmniKVMulLM(SHAPE, _config(selector_cls, bool(offload))).float()
+        lm.init_weights(seed=11, std=0.08)
+        return lm.to(torch.bfloat16).to(DEV)
+
+    def prime(lm):
+        """Prefill, then the three non-static steps in which the window still overlaps the prompt."""
+        logits, cache = lm.forward(ids, None, max_new_tokens=32, **kw)
+        tok = logits[:, -1].argmax(-1, keepdim=True)
+        for _ in range(3):
+            logits, cache = lm.forward(tok, cache)
+            tok = logits[:, -1].argmax(-1, keepdim=True)
+        return cache, tok
+
+    # eager static steps
+    lm = fresh()
+    cache, tok = prime(lm)
+    cache.enable_static_decode()
+    fused = _CallCounter(monkeypatch, "dense_attn_window")
+    eager = []
+    for _ in range(steps + 2):
+        logits, cache = lm.forward(tok, cache)
+        tok = logits[:, -1].argmax(-1, keepdim=True)
+        eager.append((logits.clone(), int(tok)))
+    assert fused.calls == 2 * (steps + 2)
+    # the same steps: two eager static ones (capture_decode's warm-up), then replays
+    lm2 = fresh()
+    cache2, tok2 = prime(lm2)
+    graph, token, glogits = lm2.capture_decode(cache2, tok2, warmup=2)
+    assert fused.calls == 2 * (steps + 2) + 2 * 3  # two warm-up steps and the captured one
+    assert int(token) == eager[1][1]
+    for t in range(steps):
+        graph.replay()
+        torch.cuda.synchronize()
+        _ = (glogits.clone() * 2).sum().item()
+        assert torch.equal(glogits, eager[2 + t][0]), t
+        assert int(token) == eager[2 + t][1], t
+    assert fused.calls == 2 * (steps + 2) + 2 * 3  # replays run the captured launches, not Python
 
 
 @pytest.mark.parametrize("selector_cls,offload", [("last", False), ("softmax_before_last", False), ("last", True),

@@ -84,6 +84,20 @@ def test_library_exports_every_declared_symbol():
     assert lib.okv_strerror(-3) == b"workspace too small"
 
 
+def test_measurement_hooks_live_in_the_measurement_build_only():
+    """The product library holds the public interface and nothing of the okv_diag_* hooks (a process-wide
+    switch that makes entry points skip their merge has no place in a serving process); the measurement
+    build next to it holds both."""
+    import ctypes as C
+    hooks = ("okv_diag_split_pass_only", "okv_diag_split_geometry", "okv_diag_gather_floor", "okv_diag_empty_launch")
+    product = C.CDLL(_lib.LIB_PATH)
+    for name in hooks:
+        assert not hasattr(product, name), name
+    diag = C.CDLL(_lib.DIAG_LIB_PATH)
+    for name in hooks + tuple(_lib.EXPORTS):
+        assert getattr(diag, name) is not None
+
+
 def test_header_is_plain_c(tmp_path):
     """The boundary is a C ABI: the header must compile as C99 and as C++ with nothing but the
     standard headers (no torch, no HIP types in the signatures)."""
@@ -212,8 +226,15 @@ def test_config_get_sets_and_returns_default():
     assert cfg.get("window_size", 16) == 16
     assert cfg.window_size == 16  # omnikv_config.py:15-19: the default is written back
     assert okv_cache.get_cache_cls(cfg) is okv_cache.OmniKVMultiStageCache
-    with pytest.raises(NotImplementedError):
-        okv_cache.get_cache_cls(okv_config.OmniKVConfig(cache_cls="lazy"))
+    # `lazy` (modeling/spec_cache.py:523-557) is the multi-stage cache with re-selection skipping at 0.4
+    lazy = okv_cache.get_cache_cls(okv_config.OmniKVConfig(cache_cls="lazy"))
+    assert issubclass(lazy, okv_cache.OmniKVMultiStageCache)
+    assert lazy([0, 4], 4, 1, False).skip_threshold == 0.4
+    assert lazy([0, 4], 4, 1, False, skip_threshold=0.7).skip_threshold == 0.7
+    assert okv_cache.OmniKVMultiStageCache([0, 4], 4, 1, False).skip_threshold is None
+    for other in ("default", "eff"):  # other model paths of the reference
+        with pytest.raises(NotImplementedError):
+            okv_cache.get_cache_cls(okv_config.OmniKVConfig(cache_cls=other))
 
 
 def test_cache_schedule_matches_oracle():

@@ -289,6 +289,37 @@ def test_per_kv_head_evaluation_equals_the_whole_tensor_functions(sel):
     assert torch.allclose(orc.gqa_attention_by_kv_head(q, k, v), orc.gqa_attention(q, k, v), rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("sel", ["uniform", "exp"])
+@pytest.mark.parametrize("w,hq,hkv", [(1, 8, 8), (5, 32, 8), (16, 32, 8), (7, 16, 4)])
+def test_window_scores_per_kv_head_equal_the_position_loop(sel, w, hq, hkv):
+    """score_window_by_kv_head against score_tokens (the reference's position-by-position loop over
+    all q heads at once), and against a brute-force evaluation in float64 with Python loops over
+    positions and heads on a tiny case: a dropped position, a wrong decay or a head max taken
+    over the wrong axis fails."""
+    g = torch.Generator().manual_seed(40 + w)
+    q = torch.randn((2, hq, w, 128), generator=g)
+    k = torch.randn((2, hkv, 300, 128), generator=g)
+    k[:, :, 0] *= 3.0
+    whole = orc.score_tokens(q, k, 257, sel)
+    by_head = orc.score_window_by_kv_head(q, k, 257, sel)
+    assert by_head.shape == whole.shape == (2, 257)
+    assert torch.allclose(by_head, whole, rtol=2e-5, atol=2e-5 * float(whole.abs().max()))
+    # brute force, float64: score[t] = sum_w weight_w * max_h softmax_t(q_hw . k_t / sqrt(D))
+    n = 23
+    qd, kd = q[:1].double(), k[:1, :, :n].double()
+    grp = hq // hkv
+    want = torch.zeros(n, dtype=torch.float64)
+    for wi in range(w):
+        best = torch.zeros(n, dtype=torch.float64)
+        for h in range(hq):
+            logit = torch.stack([(qd[0, h, wi] * kd[0, h // grp, t]).sum() / 128 ** 0.5 for t in range(n)])
+            best = torch.maximum(best, torch.softmax(logit, dim=0))
+        weight = 1.0 if sel == "uniform" else 2.0 ** (wi - w + 1)
+        want += weight * best
+    got = orc.score_window_by_kv_head(q[:1], k[:1], n, sel)[0].double()
+    assert torch.allclose(got, want, rtol=1e-5, atol=1e-7)
+
+
 def test_paged_rows_round_trip_with_loops():
     """Scatter a request into a shuffled pool token by token with Python loops; paged_rows
     must read back exactly the original rows, for page sizes 1 (token slots), 4 and 16."""
