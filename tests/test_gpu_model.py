@@ -145,37 +145,62 @@ class _CallCounter:
 def test_greedy_decode_bf16_window_selectors_take_the_fused_filter_layer(selector_cls, real_offload, monkeypatch):
     """The 16-bit model path of the window selectors: the filter layer's attention and its first scoring
     pass are one call (okv_dense_attn_window), through the steps in which the window still overlaps the
-    prompt (forced positions appended) and beyond.  Reference: the oracle runner in fp32 on the same
-    bf16-rounded weights, teacher-forced.  bf16 activations round differently from fp32 ones, so logits are
-    compared within 3% of their range and tokens wherever the oracle's top two are further apart than that."""
+    prompt (forced positions appended) and beyond.  Two references, teacher-forced with the first one's tokens:
+    the same bf16 model with the fused call switched off (selection and attention as separate calls: the same
+    bf16 roundings everywhere, only partial sums grouped differently -- tight), and the oracle runner in fp32
+    on the same bf16-rounded weights (bf16 activations against fp32 ones through seven layers -- loose)."""
+    from omnikv_amd import ops
     torch.manual_seed(0)
-    cfg = _config(selector_cls, real_offload)
-    lm = OmniKVMulLM(SHAPE, cfg).float()
-    lm.init_weights(seed=3, std=0.08)
-    lm = lm.to(torch.bfloat16)
-    ref = _OracleRunner(copy.deepcopy(lm).float(), _config(selector_cls, real_offload))
-    dut = lm.to(DEV)
-    fused = _CallCounter(monkeypatch, "dense_attn_window")
+
+    def fresh():
+        lm = OmniKVMulLM(SHAPE, _config(selector_cls, real_offload)).float()
+        lm.init_weights(seed=3, std=0.08)
+        return lm.to(torch.bfloat16)
+
+    ref = _OracleRunner(copy.deepcopy(fresh()).float(), _config(selector_cls, real_offload))
     n, steps = 500, 7  # window_size 4: steps 1..3 append forced prompt positions, 4.. do not
     ids = torch.randint(0, SHAPE.vocab_size, (1, n), generator=torch.Generator().manual_seed(1))
+
+    # the separate path first: window_supported() says no, select_with_query + attend run
+    with monkeypatch.context() as mp:
+        mp.setattr(ops, "window_supported", lambda q, k: False)
+        fused_off = _CallCounter(mp, "dense_attn_window")
+        plain = fresh().to(DEV)
+        logits, cache = plain.forward(ids.to(DEV), None, max_new_tokens=16)
+        separate = [logits.clone()]
+        toks = []
+        for t in range(steps):
+            toks.append(separate[-1][:, -1].argmax(-1, keepdim=True))
+            logits, cache = plain.forward(toks[-1], cache)
+            separate.append(logits.clone())
+        assert fused_off.calls == 0
+        if real_offload:
+            cache._join_worker()
+
+    fused = _CallCounter(monkeypatch, "dense_attn_window")
+    dut = fresh().to(DEV)
     want = ref.forward(ids)
     got, cache = dut.forward(ids.to(DEV), None, max_new_tokens=16)
     scale = float(want.abs().max())
-    assert (got.cpu() - want).abs().max() < 0.03 * scale
-    agree = checked = 0
+    assert torch.equal(got, separate[0])  # the prefill does not select
+    assert (got.cpu() - want).abs().max() < 0.1 * scale
     for t in range(steps):
-        tok = want[:, -1].argmax(-1, keepdim=True)
-        want = ref.forward(tok)
-        got, cache = dut.forward(tok.to(DEV), cache)
-        assert (got.cpu() - want).abs().max() < 0.03 * scale, (selector_cls, real_offload, t)
+        want = ref.forward(toks[t].cpu())
+        got, cache = dut.forward(toks[t], cache)
+        # fused against separate: the window scores agree to ~2e-5 (other split grouping), so the selections
+        # are the same up to near-ties and the logits to bf16 rounding of a few attention outputs
+        assert (got - separate[t + 1]).abs().max() < 0.02 * scale, (selector_cls, real_offload, t)
+        assert int(got[0, 0].argmax()) == int(separate[t + 1][0, 0].argmax()) or \
+            float(separate[t + 1][0, 0].topk(2).values.diff().abs()) < 0.04 * scale
+        assert (got.cpu() - want).abs().max() < 0.1 * scale, (selector_cls, real_offload, t)
         top2 = want[0, 0].topk(2).values
-        if float(top2[0] - top2[1]) > 0.06 * scale:
-            checked += 1
-            agree += int(got[0, 0].argmax()) == int(want[0, 0].argmax())
-    assert agree == checked
+        if float(top2[0] - top2[1]) > 0.2 * scale:
+            assert int(got[0, 0].argmax()) == int(want[0, 0].argmax())
     assert fused.calls == 2 * steps  # both filter layers, every decode step
     sel = cache._idx[1]
     assert sel.dtype == torch.int32 and sel.shape[1] == int(0.1 * n)  # forced window gone: k rows again
+    if real_offload:
+        cache._join_worker()
 
 
 def test_generate_greedy_and_error_paths():
@@ -236,7 +261,8 @@ def test_graph_replayed_bf16_window_decode_takes_the_fused_branch(selector_cls, 
     lm2 = fresh()
     cache2, tok2 = prime(lm2)
     graph, token, glogits = lm2.capture_decode(cache2, tok2, warmup=2)
-    assert fused.calls == 2 * (steps + 2) + 2 * 3  # two warm-up steps and the captured one
+    after_capture = 2 * (steps + 2) + 2 * 3 + 2 * 3  # + the second model's three priming steps, two warm-up steps and the captured one
+    assert fused.calls == after_capture
     assert int(token) == eager[1][1]
     for t in range(steps):
         graph.replay()
@@ -244,7 +270,7 @@ def test_graph_replayed_bf16_window_decode_takes_the_fused_branch(selector_cls, 
         _ = (glogits.clone() * 2).sum().item()
         assert torch.equal(glogits, eager[2 + t][0]), t
         assert int(token) == eager[2 + t][1], t
-    assert fused.calls == 2 * (steps + 2) + 2 * 3  # replays run the captured launches, not Python
+    assert fused.calls == after_capture  # replays run the captured launches, not Python
 
 
 @pytest.mark.parametrize("selector_cls,offload", [("last", False), ("softmax_before_last", False), ("last", True),
