@@ -98,7 +98,7 @@ def _declare(l):
         l.okv_diag_split_geometry.restype = C.c_int
         l.okv_diag_split_geometry.argtypes = [C.c_int, C.POINTER(Shape), C.POINTER(i32), C.POINTER(i32)]
         l.okv_diag_gather_floor.restype = C.c_int
-        l.okv_diag_gather_floor.argtypes = [vp, vp, C.POINTER(KVLayout), vp, i32, i32, i32, vp, vp]
+        l.okv_diag_gather_floor.argtypes = [vp, vp, C.POINTER(KVLayout), vp, i64, vp, i32, i32, i32, i32, vp, vp]
         l.okv_diag_empty_launch.restype = C.c_int
         l.okv_diag_empty_launch.argtypes = [vp, vp]
     l.okv_score.restype = C.c_int

@@ -117,10 +117,13 @@ constexpr int kWindowLdsFloats = 2 * 16 * kWinCols;  // [16 lane rows][64 column
 // k_rows_to_a_operand); the gather modes keep the direct A-operand loads: their pass is a
 // chain of latencies and the detour adds to it (measured: 13.5 vs 13.1 us at 8781 rows).
 __host__ __device__ constexpr bool stage1_k_through_lds(int mode) { return mode == 0 || mode == 3; }
+__host__ __device__ constexpr bool stage1_gathers(int mode) { return mode == 1 || mode == 4; }  // main rows + tail, two "tokens" per lane
 
 // MODE 0: contiguous rows, no index, no tail.  MODE 1: rows through idx (no page table),
 // optional tail.  MODE 2: anything (page tables, idx or not, tail or not).  MODE 3: page
 // table with pages of 2^n >= 16 rows, no index, no tail (a tile never straddles a page).
+// MODE 4: contiguous rows followed by a tail (selected rows staged from the host tier): MODE 1
+// with the row number in place of the index lookup.
 // WINDOW: the tiles of the scored splits also meet the W x G window query rows of the kv head
 // (four more 16-column B operands: column c is position c / G, q head g*G + c % G) and every
 // column keeps the running max and sum of its logits; nothing else changes.
@@ -194,17 +197,18 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
   // issued from clamped positions, so every tile has the same loads in flight; a row of the tail
   // segment is carried as the complement of its position there (negative).  Tiles that lie wholly
   // inside the selected rows of the split take the short address arithmetic.
-  const int direct_end = MODE == 1 ? min(main_len, end) : 0;
+  constexpr bool GATHERS = stage1_gathers(MODE);
+  const int direct_end = GATHERS ? min(main_len, end) : 0;
   auto gather_tok = [&](int r) -> int32_t {
     r = r < last ? r : last;
     int ri = r < main_len ? r : main_len - 1;
     ri = ri < 0 ? 0 : ri;  // a request with tail rows only: the index still holds one entry
-    const int32_t t = idx_row[ri];
+    const int32_t t = MODE == 1 ? idx_row[ri] : ri;
     const int32_t in_tail = (main_len - 1 - r) >> 31;  // all ones for a tail row
     return t ^ ((t ^ ~(r - main_len)) & in_tail);
   };
   auto tile_rows = [&](int tbase, TileRows& tr) {
-    if (MODE == 1) {
+    if (GATHERS) {
       tr.direct = __builtin_amdgcn_readfirstlane(tbase) + 16 <= direct_end;
       tr.tok[0] = gather_tok(tbase + r16);
       tr.tok[1] = gather_tok(tbase + 4 * j4 + (r16 & 3));
@@ -251,7 +255,7 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
     return (is_v ? vb : kb) + (uint64_t)(uint32_t)tr.tok[x] * ts;
   };
   auto load_tile = [&](const TileRows& tr, uint4 (&kf)[4], uint4 (&vf)[4]) {
-    if (MODE == 1) {
+    if (GATHERS) {
       // a row's address from its (possibly complemented) token: selected rows of K / V, or rows of the tail
       auto addr = [&](int32_t e, bool is_v) -> const T* {
         const bool in_tail = e < 0;
@@ -614,6 +618,7 @@ static void launch_g(const void* q, const RowList& rows, int hq, int hkv, int ba
   if (!rows.idx && !rows.page_table && no_tail) mode = 0;
   else if (rows.idx && !rows.page_table && rows.max_main_len >= 1) mode = 1;
   else if (rows.page_table && !rows.idx && no_tail && rows.page_shift >= 4) mode = 3;
+  else if (!rows.idx && !rows.page_table && with_v && !write_logits) mode = 4;  // contiguous rows + tail
 #define OKV_MODES(WV, LG)                                                                  \
   do {                                                                                     \
     if (mode == 0) launch_one<T, G, WV, 0, LG>(q, rows, hq, hkv, batch, scale, w, stream); \
@@ -621,7 +626,8 @@ static void launch_g(const void* q, const RowList& rows, int hq, int hkv, int ba
     else if (mode == 3) launch_one<T, G, WV, 3, LG>(q, rows, hq, hkv, batch, scale, w, stream); \
     else launch_one<T, G, WV, 2, LG>(q, rows, hq, hkv, batch, scale, w, stream);           \
   } while (0)
-  if (!with_v) OKV_MODES(false, true);  // scoring only
+  if (mode == 4) launch_one<T, G, true, 4, false>(q, rows, hq, hkv, batch, scale, w, stream);
+  else if (!with_v) OKV_MODES(false, true);  // scoring only
   else if (write_logits) OKV_MODES(true, true);
   else OKV_MODES(true, false);
 #undef OKV_MODES

@@ -13,12 +13,17 @@ namespace okv {
 // load of up to four tiles in flight at once, and no arithmetic beyond an XOR of what arrived.
 template <int TILES>
 __global__ __launch_bounds__(256) void gather_floor_kernel(const char* __restrict__ kb, const char* __restrict__ vb,
-                                                           const int32_t* __restrict__ idx, int sel_len,
+                                                           const int32_t* __restrict__ idx_all, int64_t idx_stride,
+                                                           const int32_t* __restrict__ sel_lens, int max_sel_len,
                                                            int split_rows, int64_t token_bytes, int64_t head_bytes,
-                                                           uint32_t* __restrict__ sink) {
-  const int g = blockIdx.x, split = blockIdx.y;
+                                                           int64_t batch_bytes, uint32_t* __restrict__ sink) {
+  const int g = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, j4 = lane >> 4;
+  const int sel_len = sel_lens ? sel_lens[b] : max_sel_len;
+  const int32_t* idx = idx_all + (int64_t)b * idx_stride;
+  kb += (int64_t)b * batch_bytes;
+  vb += (int64_t)b * batch_bytes;
   const int begin = split * split_rows, end = min(begin + split_rows, sel_len);
   if (begin >= end) return;
   const int last = end - 1;
@@ -87,25 +92,27 @@ int okv_diag_split_geometry(int op, const okv_shape_t* s, int32_t* split_rows, i
   return OKV_OK;
 }
 
-// The load-only counterpart of one okv_sparse_attn launch over rows idx[0 .. sel_len) of a
-// contiguous batch-1 K / V (no tail): same grid (kv heads x splits of split_rows rows), same
-// bytes; a wave keeps the loads of tiles_in_flight (1, 2 or 4) of its tiles outstanding.  sink: 4 bytes
-// of device memory.
+// The load-only counterpart of one okv_sparse_attn launch over rows idx[b][0 .. sel_len_b) of contiguous K / V
+// or of a pool addressed as token slots (no tail): same grid (kv heads x splits of split_rows rows x requests),
+// same bytes; a wave keeps the loads of tiles_in_flight (1, 2 or 4) of its tiles outstanding.  sel_lens: device
+// int32[batch] or NULL.  sink: 4 bytes of device memory.
 int okv_diag_gather_floor(const void* k_base, const void* v_base, const okv_kv_layout_t* layout,
-                          const int32_t* idx, int32_t sel_len, int32_t split_rows, int32_t tiles_in_flight,
-                          void* sink, okv_stream_t stream) {
+                          const int32_t* idx, int64_t idx_stride, const int32_t* sel_lens, int32_t max_sel_len,
+                          int32_t batch, int32_t split_rows, int32_t tiles_in_flight, void* sink,
+                          okv_stream_t stream) {
   int rc = validate_layout(layout, k_base, v_base);
   if (rc) return rc;
-  OKV_REQUIRE(idx && sink && sel_len >= 1, OKV_ERR_INVALID, "idx, sink or sel_len");
+  OKV_REQUIRE(idx && sink && max_sel_len >= 1 && batch >= 1, OKV_ERR_INVALID, "idx, sink, max_sel_len or batch");
   OKV_REQUIRE(split_rows >= 16 && split_rows % 16 == 0, OKV_ERR_INVALID, "split_rows must be a multiple of 16");
   OKV_REQUIRE(layout->page_table == nullptr && layout->dtype != OKV_F32, OKV_ERR_UNSUPPORTED,
               "the floor kernel reads contiguous 16-bit K/V");
   OKV_REQUIRE(tiles_in_flight == 1 || tiles_in_flight == 2 || tiles_in_flight == 4, OKV_ERR_INVALID,
               "tiles_in_flight must be 1, 2 or 4");
-  dim3 grid(layout->num_kv_heads, (sel_len + split_rows - 1) / split_rows);
+  dim3 grid(layout->num_kv_heads, (max_sel_len + split_rows - 1) / split_rows, batch);
   auto kern = tiles_in_flight == 1 ? gather_floor_kernel<1> : tiles_in_flight == 2 ? gather_floor_kernel<2> : gather_floor_kernel<4>;
   hipLaunchKernelGGL(kern, grid, dim3(256), 0, (hipStream_t)stream, (const char*)k_base, (const char*)v_base, idx,
-                     sel_len, split_rows, layout->token_stride * 2, layout->head_stride * 2, (uint32_t*)sink);
+                     idx_stride, sel_lens, max_sel_len, split_rows, layout->token_stride * 2, layout->head_stride * 2,
+                     layout->batch_stride * 2, (uint32_t*)sink);
   OKV_HIP_CHECK(hipGetLastError());
   return OKV_OK;
 }

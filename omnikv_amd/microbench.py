@@ -140,9 +140,9 @@ def main():
         l = i % nl
         if args.op == "sparse_floor":
             rows, sink, lay, C = floor
-            return check(lib().okv_diag_gather_floor(ks[l].data_ptr(), vs[l].data_ptr(), C.byref(lay), idx.data_ptr(), k_sel,
-                                                     rows, args.tiles_in_flight, sink.data_ptr(),
-                                                     torch.cuda.current_stream().cuda_stream))
+            return check(lib().okv_diag_gather_floor(ks[l].data_ptr(), vs[l].data_ptr(), C.byref(lay), idx.data_ptr(),
+                                                     idx.stride(0), None, k_sel, 1, rows, args.tiles_in_flight,
+                                                     sink.data_ptr(), torch.cuda.current_stream().cuda_stream))
         if args.op == "empty":
             return check(lib().okv_diag_empty_launch(floor[1].data_ptr(), torch.cuda.current_stream().cuda_stream))
         if args.op == "dense":
