@@ -75,9 +75,14 @@ static int choose_split_rows(int batch, int hq, int hkv, int total_rows, bool wi
   auto plan = [&](int per_cu, int64_t logit_bytes, int64_t* rounds_out) -> int {
     const int64_t capacity = (int64_t)num_compute_units() * per_cu;
     const int64_t cap_rows = with_logits ? std::min<int64_t>(logit_bytes / (4 * group) / 64 * 64, 8192) : kind == 2 ? 8192 : 4096;
+    // a sparse layer's share is a few 16-row tiles per wave: cut to the tile, so that all CUs hold two
+    // workgroups (137 -> 144 rows at 8781 selected rows, where rounding to 64 left 112 CUs with two
+    // workgroups of 192 and 144 CUs with one)
+    const int64_t gran = kind == 1 && batch <= 1 ? 16 : 64;
     for (int64_t rounds = 1;; ++rounds) {
       int64_t rows = (work + rounds * capacity - 1) / (rounds * capacity);
-      rows = (rows + 63) / 64 * 64;
+      rows = (rows + gran - 1) / gran * gran;
+      if (rows < 64) rows = 64;
       if (rounds == 1 && with_v && batch > 1 && rows <= 128) {
         // a short pass is a chain of latencies: fewer, fatter workgroups
         rows = (work + capacity * 2 / 3 - 1) / (capacity * 2 / 3);

@@ -8,7 +8,7 @@
 namespace okv {
 
 // What a kernel that ONLY fetches the rows of a sparse layer costs: the grid, the row -> wave
-// assignment, the index lookup and the two load shapes of attn_stage1_mfma's gather mode (K:
+// assignment, the index lookups and the two load shapes of attn_stage1_mfma's gather mode (K:
 // lane = row, 4 x 16 bytes of each 64-byte k-step; V: whole 256-byte rows per 16 lanes), every
 // load of up to four tiles in flight at once, and no arithmetic beyond an XOR of what arrived.
 template <int TILES>
@@ -31,13 +31,14 @@ __global__ __launch_bounds__(256) void gather_floor_kernel(const char* __restric
   const char* vh = vb + (int64_t)g * head_bytes;
   uint32_t acc = 0;
   for (int t0 = begin + wave * 16; t0 < end; t0 += 64 * TILES) {
-    int tk[TILES], tv[TILES][4];
+    // two lookups per lane and tile, as the kernel does: the lane's K row (tile row r16) and one of its lane
+    // row's four V rows (tile row 4*j4 + r16%4; the quad holds the four between its lanes)
+    int tk[TILES], tq[TILES];
 #pragma unroll
     for (int d = 0; d < TILES; ++d) {
       const int tb = min(t0 + 64 * d, last);  // a tile past the wave's share repeats its last row (as the kernel clamps)
       tk[d] = idx[min(tb + r16, last)];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) tv[d][i] = idx[min(tb + 4 * j4 + i, last)];
+      tq[d] = idx[min(tb + 4 * j4 + (r16 & 3), last)];
     }
     uint4 a[TILES][4], b[TILES][4];
 #pragma unroll
@@ -46,9 +47,11 @@ __global__ __launch_bounds__(256) void gather_floor_kernel(const char* __restric
       const char* p = kh + (int64_t)tk[d] * token_bytes + 16 * j4;
 #pragma unroll
       for (int s = 0; s < 4; ++s) a[d][s] = *reinterpret_cast<const uint4*>(p + 64 * s);
+      const int tv[4] = {__builtin_amdgcn_update_dpp(0, tq[d], 0x00, 0xf, 0xf, true), __builtin_amdgcn_update_dpp(0, tq[d], 0x55, 0xf, 0xf, true),
+                         __builtin_amdgcn_update_dpp(0, tq[d], 0xaa, 0xf, 0xf, true), __builtin_amdgcn_update_dpp(0, tq[d], 0xff, 0xf, 0xf, true)};
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        b[d][i] = load_stream16(vh + (int64_t)tv[d][i] * token_bytes + 16 * r16);
+        b[d][i] = load_stream16(vh + (int64_t)tv[i] * token_bytes + 16 * r16);
     }
 #pragma unroll
     for (int d = 0; d < TILES; ++d) {

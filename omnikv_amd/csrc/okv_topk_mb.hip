@@ -52,6 +52,15 @@ struct TopkMbWs {
   int chunk_tiles;
 };
 
+// all arguments of a launch in one batch of scalar loads at the top (see fetch_now)
+__device__ __forceinline__ void fetch_topk_args_now(const float* scores, int64_t score_stride, const int32_t* seq_lens,
+                                                    int max_seq_len, const int32_t* k_per_seg, int max_k,
+                                                    const TopkMbWs& w) {
+  fetch_now(scores); fetch_now(score_stride); fetch_now(seq_lens); fetch_now(max_seq_len); fetch_now(k_per_seg);
+  fetch_now(max_k); fetch_now(w.hist0); fetch_now(w.coarse); fetch_now(w.cand); fetch_now(w.cand_base);
+  fetch_now(w.chunk_gt); fetch_now(w.state); fetch_now(w.max_chunks); fetch_now(w.chunk_tiles);
+}
+
 static void chunking(int max_seq_len, int* chunk_tiles, int* chunks) {
   const int tiles = (max_seq_len + kTile - 1) / kTile;
   int ct = (tiles + kTargetChunks - 1) / kTargetChunks;
@@ -198,6 +207,7 @@ __global__ __launch_bounds__(kMbThreads) void topk_mb_hist(const float* __restri
                                                            int max_seq_len,
                                                            const int32_t* __restrict__ k_per_seg,
                                                            int max_k, TopkMbWs w) {
+  fetch_topk_args_now(scores, score_stride, seq_lens, max_seq_len, k_per_seg, max_k, w);
   __shared__ __attribute__((aligned(16))) uint32_t lh[kBins12];
   const int c = blockIdx.x, b = blockIdx.y, t = threadIdx.x;
   const int n = req_len(seq_lens, max_seq_len, b);
@@ -246,6 +256,7 @@ __global__ __launch_bounds__(kMbThreads) void topk_mb_cand(const float* __restri
                                                            int max_seq_len,
                                                            const int32_t* __restrict__ k_per_seg,
                                                            int max_k, TopkMbWs w) {
+  fetch_topk_args_now(scores, score_stride, seq_lens, max_seq_len, k_per_seg, max_k, w);
   __shared__ __attribute__((aligned(16))) uint32_t ch[256];  // the request's 256-bin summary
   __shared__ uint32_t fh[16];   // its 16 fine bins inside the summary bin of the k-th key
   __shared__ uint32_t fhb[16];  // the same over the chunks before this one
@@ -367,6 +378,9 @@ __global__ __launch_bounds__(kMbThreads) void topk_mb_write(const float* __restr
                                                             int max_k, TopkMbWs w,
                                                             int32_t* __restrict__ idx_out,
                                                             int64_t idx_stride) {
+  fetch_topk_args_now(scores, score_stride, seq_lens, max_seq_len, k_per_seg, max_k, w);
+  fetch_now(idx_out);
+  fetch_now(idx_stride);
   __shared__ __attribute__((aligned(16))) uint32_t hA[1024], hB[1024], hBb[1024];
   __shared__ uint32_t cache[kCandCache];
   __shared__ uint32_t sm[8];
