@@ -41,7 +41,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dense split pass from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE
 # (profiles/dense_split_pass_pmc.txt), keyed by (context, tail, dtype); None when not measured.
-TRAFFIC_BYTES = {(131072, 1, "bf16"): 537.1e6 + 1.04e6}
+TRAFFIC_BYTES = {(131072, 1, "bf16"): 537.1e6 + 1.04e6, (450000, 1, "bf16"): 1843.4e6 + 2.11e6}
 HQ, HKV, D, LAYERS = 32, 8, 128, 32
 FILTER_LAYERS = (2, 8, 18)
 WAIT = 1

@@ -12,6 +12,7 @@ import os
 _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "libomnikv_hip.so")
 DIAG_LIB_PATH = os.path.join(_PKG, "libomnikv_hip_diag.so")  # measurement build: + the okv_diag_* hooks
+STAMPS_LIB_PATH = os.path.join(_PKG, "libomnikv_hip_stamps.so")  # timeline build (csrc/build.py --stamps): + device timestamps
 
 OKV_F32, OKV_BF16, OKV_F16 = 0, 1, 2
 OKV_REDUCE_MAX, OKV_REDUCE_SUM = 0, 1
@@ -101,6 +102,9 @@ def _declare(l):
         l.okv_diag_gather_floor.argtypes = [vp, vp, C.POINTER(KVLayout), vp, i64, vp, i32, i32, i32, i32, vp, vp]
         l.okv_diag_empty_launch.restype = C.c_int
         l.okv_diag_empty_launch.argtypes = [vp, vp]
+    if hasattr(l, "okv_stamps_read"):  # the timeline build only
+        l.okv_stamps_read.restype = C.c_int
+        l.okv_stamps_read.argtypes = [C.c_int, vp, C.c_int]
     l.okv_score.restype = C.c_int
     l.okv_score.argtypes = [vp, vp, C.POINTER(KVLayout), vp, i32, i32, i32, i32, f32, vp, i64, vp, sz, vp]
     l.okv_score_window.restype = C.c_int
@@ -143,20 +147,21 @@ def _declare(l):
 _want_diag = False
 
 
-def use_diag_build() -> None:
+def use_diag_build(stamps: bool = False) -> None:
     """Benchmarks call this before anything else touches the library: the process then loads the
-    measurement build (the product's sources + the okv_diag_* hooks) instead of the product library."""
+    measurement build (the product's sources + the okv_diag_* hooks) instead of the product library;
+    stamps=True: the timeline build (measurement build + device timestamps in two kernels)."""
     global _want_diag
     if _lib is not None and not hasattr(_lib, "okv_diag_split_pass_only"):
         raise OmniKVLibraryError("the product library is already loaded: call use_diag_build() first")
-    _want_diag = True
+    _want_diag = "stamps" if stamps else True
 
 
 def lib():
     """The loaded library; raises if it has not been built."""
     global _lib
     if _lib is None:
-        path = DIAG_LIB_PATH if _want_diag else LIB_PATH
+        path = STAMPS_LIB_PATH if _want_diag == "stamps" else DIAG_LIB_PATH if _want_diag else LIB_PATH
         if not os.path.exists(path):
             raise OmniKVLibraryError(
                 f"{path} is missing: build it with `python omnikv_amd/csrc/build.py` "

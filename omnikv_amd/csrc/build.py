@@ -5,7 +5,11 @@
                                     okv_diag.hip (split-pass-only switch, load-only floor kernel, empty
                                     launch); loaded by bench.py and omnikv_amd.microbench only
 
-Usage: python omnikv_amd/csrc/build.py [--no-diag]
+  omnikv_amd/libomnikv_hip_stamps.so  only with --stamps: the measurement build plus device timestamps inside the
+                                      gather-mode split pass and the merge (-DOKV_STAMPS), for
+                                      `python -m omnikv_amd.microbench --op sparse_timeline`
+
+Usage: python omnikv_amd/csrc/build.py [--no-diag] [--stamps]
 """
 import os
 import subprocess
@@ -15,6 +19,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
 OUT = os.path.join(PKG, "libomnikv_hip.so")
 OUT_DIAG = os.path.join(PKG, "libomnikv_hip_diag.so")
+OUT_STAMPS = os.path.join(PKG, "libomnikv_hip_stamps.so")
 SOURCES = ["okv_api.hip", "okv_attn.hip", "okv_attn_mfma.hip", "okv_topk.hip", "okv_topk_mb.hip", "okv_gather.hip",
            "okv_window.hip", "okv_layer.hip"]
 DIAG_SOURCES = SOURCES + ["okv_diag.hip"]
@@ -43,6 +48,11 @@ def _compile(sources, out, extra, verbose):
     if res.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + text)
     return out
+
+
+def build_stamps(verbose: bool = True) -> str:
+    """The timeline build (not part of build(): nothing loads it but microbench --op sparse_timeline)."""
+    return _compile(DIAG_SOURCES, OUT_STAMPS, ["-DOKV_DIAG", "-DOKV_STAMPS"], verbose)
 
 
 def build(force: bool = True, verbose: bool = True, diag: bool = True) -> str:
@@ -80,6 +90,9 @@ def build_abi_smoke(verbose: bool = True) -> str:
 
 
 if __name__ == "__main__":
+    if "--stamps" in sys.argv:
+        print("built", build_stamps())
+        sys.exit(0)
     build(force=True, diag="--no-diag" not in sys.argv)
     print("built", OUT, "" if "--no-diag" in sys.argv else "and " + OUT_DIAG)
     print("built", build_abi_smoke())

@@ -152,6 +152,9 @@ __global__ __launch_bounds__(256) void attn_stage1_generic(const T* __restrict__
 }
 
 // ------------------------------------------------------------------- merge
+#ifdef OKV_STAMPS
+__device__ unsigned long long g_merge_stamps[kStampBlocks * kStampSlots];
+#endif
 // grid (q heads, batch), 256 threads: 32 float4 columns x 8 split lanes.  Every
 // thread folds its splits with a running max (all loads independent, one trip to
 // memory), then the 8 split lanes of a column meet in LDS.
@@ -160,6 +163,7 @@ __device__ __forceinline__ void merge_body(const RowList& rows, int hq, const At
                                            T* __restrict__ out, int with_v, int with_score_lse, int h,
                                            int b) {
   __shared__ float4 snum[8][32];
+  OKV_STAMP(g_merge_stamps, h, 0);  // merge timeline: 0 entry, 1 arguments and lengths there, 2 own splits folded, 3 after the barrier, 4 end
   __shared__ float sm[8], sden[8], smA[8], sdenA[8];
   const int tid = threadIdx.x;
   const int main_len = rl_main_len(rows, b);
@@ -172,6 +176,7 @@ __device__ __forceinline__ void merge_body(const RowList& rows, int hq, const At
   const int dq = tid & 31, sl = tid >> 5;
   const float4* po = reinterpret_cast<const float4*>(w.part_o + ph * kD) + dq;
 
+  OKV_STAMP(g_merge_stamps, h, 1);
   float m = -INFINITY, den = 0.f, mA = -INFINITY, denA = 0.f;
   float4 num = make_float4(0.f, 0.f, 0.f, 0.f);
   constexpr int U = 8;  // splits in flight per thread: all loads of a batch leave before any is used
@@ -200,11 +205,12 @@ __device__ __forceinline__ void merge_body(const RowList& rows, int hq, const At
       m = mn;
       if (s < nA) {
         const float mnA = fmaxf(mA, x);
-        denA = fmaf(denA, exp2f(mA - mnA), exp2f(x - mnA));
+        denA = fmaf(denA, __builtin_amdgcn_exp2f(mA - mnA), __builtin_amdgcn_exp2f(x - mnA));
         mA = mnA;
       }
     }
   }
+  OKV_STAMP(g_merge_stamps, h, 2);
   snum[sl][dq] = num;
   if (dq == 0) {
     sm[sl] = m;
@@ -213,6 +219,7 @@ __device__ __forceinline__ void merge_body(const RowList& rows, int hq, const At
     sdenA[sl] = denA;
   }
   __syncthreads();
+  OKV_STAMP(g_merge_stamps, h, 3);
   if (with_v && tid < kD) {
     float M = -INFINITY;
 #pragma unroll
@@ -221,7 +228,7 @@ __device__ __forceinline__ void merge_body(const RowList& rows, int hq, const At
     float a = 0.f, d = 0.f;
 #pragma unroll
     for (int x = 0; x < 8; ++x) {
-      const float f = (sm[x] == -INFINITY) ? 0.f : exp2f(sm[x] - M);
+      const float f = (sm[x] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(sm[x] - M);
       a = fmaf(sn[x * kD + tid], f, a);
       d = fmaf(sden[x], f, d);
     }
@@ -233,9 +240,10 @@ __device__ __forceinline__ void merge_body(const RowList& rows, int hq, const At
     for (int x = 0; x < 8; ++x) M = fmaxf(M, smA[x]);
     float d = 0.f;
 #pragma unroll
-    for (int x = 0; x < 8; ++x) d += (smA[x] == -INFINITY) ? 0.f : sdenA[x] * exp2f(smA[x] - M);
+    for (int x = 0; x < 8; ++x) d += (smA[x] == -INFINITY) ? 0.f : sdenA[x] * __builtin_amdgcn_exp2f(smA[x] - M);
     w.score_lse[b * hq + h] = M + log2f(d);
   }
+  OKV_STAMP(g_merge_stamps, h, 4);
 }
 
 template <typename T>
@@ -527,6 +535,23 @@ int okv_set_option(const char* name, int value) {
   set_error("unknown option %s", name);
   return OKV_ERR_INVALID;
 }
+
+#ifdef OKV_STAMPS
+// Timeline build only: copies the device timestamps of the last launches out (which: 0 split pass, 1 merge);
+// dst holds okv::kStampBlocks * okv::kStampSlots 64-bit values, 10 ns units, 0 where nothing was stamped.
+int okv_stamps_read(int which, unsigned long long* dst, int clear) {
+  OKV_REQUIRE(dst && (which == 0 || which == 1), OKV_ERR_INVALID, "which must be 0 or 1");
+  if (which == 0) return stamps_read_split(dst, clear);
+  const size_t bytes = sizeof(unsigned long long) * kStampBlocks * kStampSlots;
+  OKV_HIP_CHECK(hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_merge_stamps), bytes));
+  if (clear) {
+    void* p = nullptr;
+    OKV_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(g_merge_stamps)));
+    OKV_HIP_CHECK(hipMemset(p, 0, bytes));
+  }
+  return OKV_OK;
+}
+#endif
 
 #ifdef OKV_DIAG
 // Measurement hook of the measurement build (compiled with -DOKV_DIAG into libomnikv_hip_diag.so; the

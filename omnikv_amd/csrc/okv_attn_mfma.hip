@@ -27,6 +27,23 @@
 
 namespace okv {
 
+#ifdef OKV_STAMPS
+__device__ unsigned long long g_split_stamps[kStampBlocks * kStampSlots];
+int stamps_read_split(unsigned long long* dst, int clear) {
+  const size_t bytes = sizeof(unsigned long long) * kStampBlocks * kStampSlots;
+  OKV_HIP_CHECK(hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_split_stamps), bytes));
+  if (clear) {
+    void* p = nullptr;
+    OKV_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(g_split_stamps)));
+    OKV_HIP_CHECK(hipMemset(p, 0, bytes));
+  }
+  return OKV_OK;
+}
+#endif
+// split pass timeline (gather mode, three-tile shares): 0 entry, 1 query loads issued, 2 index loads issued,
+// 3 first tile's row loads issued, 4 all row loads issued, 5 first tile consumed, 6 last tile consumed, 7 end
+#define SPLIT_STAMP(i) do { if (MODE == 1) OKV_STAMP(g_split_stamps, blockIdx.y * gridDim.x + blockIdx.x, i); } while (0)
+
 // two fp32 -> one dword of two 16-bit elements (first argument in the low half)
 __device__ __forceinline__ uint32_t pack2(const BF16*, float a, float b) {
   f32x2_t x = {a, b};
@@ -131,6 +148,7 @@ template <typename T, int G, bool WITH_V, int MODE, bool LOGITS, bool WINDOW>
 __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const RowList& rows, int hq, float scale,
                                                  const AttnWorkspace& w, const WindowFuse& wf) {
   extern __shared__ float lds[];
+  SPLIT_STAMP(0);
   constexpr bool KLDS = stage1_k_through_lds(MODE);
   const int g = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
   const int main_len = rl_main_len(rows, b);
@@ -154,6 +172,7 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
     for (int s = 0; s < 4; ++s) qf[s] = *reinterpret_cast<const uint4*>(qp + 32 * s);
   }
 
+  SPLIT_STAMP(1);
   constexpr int WCB = WINDOW ? kWinCols / 16 : 1;
   uint4 wqf[WCB][4];
   float wm[WCB], wl[WCB];  // per column block: state of (column r16, lane row j4), max in raw units
@@ -445,12 +464,17 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
         tile_rows(t, tr0);
         tile_rows(t + 64, tr);
         tile_rows(t + 128, tr2);
+        SPLIT_STAMP(2);
         load_tile(tr0, kA, vA);
+        SPLIT_STAMP(3);
         load_tile(tr, kB, vB);
         load_tile(tr2, kC, vC);
+        SPLIT_STAMP(4);
         compute(t, kA, vA);
+        SPLIT_STAMP(5);
         compute(t + 64, kB, vB);
         compute(t + 128, kC, vC);
+        SPLIT_STAMP(6);
       } else {
         uint4 kA[4], vA[4], kB[4], vB[4];
         TileRows tr, tr0;
@@ -562,6 +586,7 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
     if (WITH_V) w.part_o[ph * kD + d] = num / den;
     if (d == 0) w.part_lse[ph] = M * sl2 + log2f(den);
   }
+  SPLIT_STAMP(7);
 }
 
 template <typename T, int G, bool WITH_V, int MODE, bool LOGITS>

@@ -161,6 +161,25 @@ __device__ __forceinline__ void fetch_args_now(const RowList& r, const AttnWorks
   fetch_now(w.split_rows); fetch_now(w.logits_stride); fetch_now(w.group_reduce); fetch_now(w.logit_heads);
 }
 
+// Device timestamps inside the gather-mode split pass and the merge, for the timeline build only
+// (-DOKV_STAMPS, libomnikv_hip_stamps.so: `build.py --stamps`; neither the product nor the measurement
+// build contains them).  Thread 0 of every workgroup stores the 100 MHz wall clock at up to eight
+// points; okv_stamps_read copies them out.
+#ifdef OKV_STAMPS
+constexpr int kStampSlots = 8, kStampBlocks = 4096;
+// `arr`: a __device__ unsigned long long[kStampBlocks * kStampSlots] of the translation unit (device symbols
+// are not shared between them)
+#define OKV_STAMP(arr, block, i)                                                                        \
+  do {                                                                                                  \
+    if (threadIdx.x == 0 && (block) < okv::kStampBlocks) arr[(block) * okv::kStampSlots + (i)] = wall_clock64(); \
+  } while (0)
+int stamps_read_split(unsigned long long* dst, int clear);  // okv_attn_mfma.hip
+#else
+#define OKV_STAMP(arr, block, i) \
+  do {                           \
+  } while (0)
+#endif
+
 // The last W query positions of every q head riding along a dense pass (window selectors): the
 // pass then also leaves, per scored split, the log-sum-exp of every (position, head) column's
 // logits, which is what the first of the window selector's two passes over K computes.

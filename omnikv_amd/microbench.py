@@ -24,9 +24,11 @@ HQ, HKV, D = 32, 8, 128
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--op", required=True,
-                    choices=["dense", "fused", "fused_select", "fused_then_topk", "score", "topk", "sparse", "sparse_packed", "sparse_floor", "empty", "gather", "copy",
+                    choices=["dense", "fused", "fused_select", "fused_then_topk", "score", "topk", "sparse", "sparse_packed", "sparse_floor", "sparse_timeline",
+                             "empty", "gather", "copy",
                              "offload_memcpy", "offload_zero_copy", "offload_incremental", "h2d", "window", "window_loop", "window_fused", "window_then_dense",
-                             "paged_dense", "paged_fused", "paged_fused_select", "paged_score", "paged_topk", "paged_sparse", "paged_sparse_slots"])
+                             "paged_dense", "paged_fused", "paged_fused_select", "paged_score", "paged_topk", "paged_sparse", "paged_sparse_slots",
+                             "paged_sparse_floor"])
     ap.add_argument("--batch", type=int, default=16, help="requests of the paged_* ops (ragged lengths 8192..32768)")
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--pages-in-order", action="store_true", help="paged_* ops: identity page table instead of shuffled")
@@ -54,7 +56,7 @@ def main():
     args = ap.parse_args()
 
     from . import _lib as okv_lib
-    okv_lib.use_diag_build()  # the product's kernels + the measurement hooks
+    okv_lib.use_diag_build(stamps=args.op == "sparse_timeline")  # the product's kernels + the measurement hooks
     check(lib().okv_set_option(b"split_rows", args.split_rows))
     check(lib().okv_set_option(b"attn_variant", args.attn_variant))
     dev = torch.device("cuda:0")
@@ -170,7 +172,7 @@ def main():
                 s = ops.score(qw[l][:, :, t:t + 1], ks[l][:, :, :n], selector="softmax_before_last")
                 acc = s if acc is None else acc + s
             return acc
-        if args.op == "sparse":
+        if args.op in ("sparse", "sparse_timeline"):
             return ops.sparse_attn(qs[l], ks[l][:, :, :n], vs[l][:, :, :n], idx=idx,
                                    tail_k=ks[l][:, :, n:], tail_v=vs[l][:, :, n:])
         if args.op == "sparse_packed":
@@ -202,6 +204,7 @@ def main():
         "window_then_dense": 2.0 * (n + tail) * row + 4.0 * n,
         "window_loop": 1.0 * n * row + 4.0 * n,
         "sparse": 2.0 * (k_sel + tail) * row + 4.0 * k_sel,
+        "sparse_timeline": 2.0 * (k_sel + tail) * row + 4.0 * k_sel,
         "sparse_packed": 2.0 * (k_sel + tail) * row,
         "sparse_floor": 2.0 * k_sel * row + 4.0 * k_sel,
         "empty": 0.0,
@@ -226,12 +229,43 @@ def main():
     res = {"op": args.op, "ctx": n, "selected": k_sel, "tail": tail, "dtype": args.dtype,
            "layout": args.layout, "us_per_call": us, "algorithmic_bytes": algo,
            "algorithmic_GBps": algo / us / 1e3 if algo else None, "frac_of_8TBps": algo / us / 1e3 / 8000.0}
+    if args.op == "sparse_timeline":
+        res["timeline_ns"] = sparse_timeline()
     if args.op.startswith("offload"):
         res.update({"layers_per_selection": nl, "host_link_GBps": algo / us / 1e3})
         if args.op == "offload_incremental":
             res.update({"overlap": args.overlap, "rows_fetched_per_layer": off.last_fetch_count(0),
                         "full_restage_bytes": 2.0 * k_sel * row * nl})
     print(json.dumps(res))
+
+
+def sparse_timeline():
+    """Device timestamps of the LAST sparse-layer call (timeline build): nanoseconds after the first workgroup's
+    entry, over the workgroups whose first wave took the three-tile path (split pass) and the q heads (merge);
+    (min, median, p90, max) per point, then the same for the intervals between consecutive points."""
+    import ctypes as C
+
+    import numpy as np
+
+    out = {}
+    for which, names in ((0, ["entry", "query loads issued", "index loads issued", "first tile's row loads issued",
+                              "all row loads issued", "first tile consumed", "last tile consumed", "end"]),
+                         (1, ["entry", "arguments and lengths there", "own splits folded", "after the barrier", "end"])):
+        buf = (C.c_ulonglong * (4096 * 8))()
+        check(lib().okv_stamps_read(which, buf, 0))
+        a = np.frombuffer(buf, dtype=np.uint64).astype(np.int64).reshape(4096, 8)[:, :len(names)]
+        a = a[(a > 0).all(axis=1)]
+        a = (a - a[:, 0].min()) * 10
+
+        def q(c):
+            return [int(c.min()), int(np.median(c)), int(np.percentile(c, 90)), int(c.max())]
+
+        d = np.diff(a, axis=1)
+        out["split_pass" if which == 0 else "merge"] = {
+            "workgroups": int(len(a)), "columns": "min, median, p90, max",
+            "at": {nm: q(a[:, i]) for i, nm in enumerate(names)},
+            "between": {f"{names[i]} -> {names[i + 1]}": q(d[:, i]) for i in range(len(names) - 1)}}
+    return out
 
 
 def paged(args, dev):
@@ -276,7 +310,19 @@ def paged(args, dev):
     idx = torch.zeros((args.batch, kmax), dtype=torch.int32, device=dev)
     ops.topk(scores, kmax, seq_lens=lens_d, k_per_seg=k_per_d, out=idx)
 
-    slots = pools[0].slot_index(idx) if args.op == "paged_sparse_slots" else None
+    slots = pools[0].slot_index(idx) if args.op in ("paged_sparse_slots", "paged_sparse_floor") else None
+    floor = None
+    if args.op == "paged_sparse_floor":
+        # the load-only counterpart of paged_sparse_slots: same grid, slot lookups, loads and bytes, no arithmetic
+        import ctypes as C
+
+        from . import _lib
+        shape = _lib.Shape(args.batch, HQ, HKV, D, kmax, 0, 0)
+        rows_, splits_ = C.c_int32(0), C.c_int32(0)
+        check(lib().okv_diag_split_geometry(_lib.OKV_OP_SPARSE_ATTN, C.byref(shape), C.byref(rows_), C.byref(splits_)))
+        pk0 = pools[0].pool_k
+        floor = (rows_.value, torch.zeros(4, dtype=torch.int32, device=dev),
+                 _lib.KVLayout(ops._DTYPES[dtype], HQ, HKV, D, pk0.stride(1), pk0.stride(2), 0, None, 0, 0, 0), C)
 
     def call(i):
         l = i % nl
@@ -292,6 +338,11 @@ def paged(args, dev):
             return score_(qs[l], pools[l], score_len=nmax, selector=args.selector, score_lens=lens_d)
         if args.op == "paged_topk":
             return ops.topk(scores, kmax, seq_lens=lens_d, k_per_seg=k_per_d, out=idx)
+        if args.op == "paged_sparse_floor":
+            rows, sink, lay, C = floor
+            return check(lib().okv_diag_gather_floor(pools[l].pool_k.data_ptr(), pools[l].pool_v.data_ptr(), C.byref(lay),
+                                                     slots.data_ptr(), slots.stride(0), k_per_d.data_ptr(), kmax, args.batch,
+                                                     rows, 4, sink.data_ptr(), torch.cuda.current_stream().cuda_stream))
         if args.op == "paged_sparse_slots":
             return ops.sparse_attn(qs[l], pools[l], slots=slots, sel_len=kmax, sel_lens=k_per_d)
         return sparse_(qs[l], pools[l], idx=idx, sel_len=kmax, sel_lens=k_per_d)
@@ -301,7 +352,8 @@ def paged(args, dev):
     algo = {"paged_dense": 2.0 * tokens * row, "paged_fused": 2.0 * tokens * row + 4.0 * tokens,
             "paged_fused_select": 2.0 * tokens * row + 4.0 * tokens + 4.0 * sel,
             "paged_score": 1.0 * tokens * row + 4.0 * tokens, "paged_topk": 4.0 * tokens + 4.0 * sel,
-            "paged_sparse": 2.0 * sel * row + 4.0 * sel, "paged_sparse_slots": 2.0 * sel * row + 4.0 * sel}[args.op]
+            "paged_sparse": 2.0 * sel * row + 4.0 * sel, "paged_sparse_slots": 2.0 * sel * row + 4.0 * sel,
+            "paged_sparse_floor": 2.0 * sel * row + 4.0 * sel}[args.op]
     for i in range(args.warmup):
         call(i)
     torch.cuda.synchronize()
