@@ -255,6 +255,21 @@ __global__ __launch_bounds__(256) void attn_merge(RowList rows, int hq, AttnWork
   merge_body<T>(rows, hq, w, out, with_v, with_score_lse, blockIdx.x, blockIdx.y);
 }
 
+// The merge launch behind a dense pass with window columns: blocks [0, Hq) of a request merge the
+// attention partials, blocks [Hq, Hq + Hkv) the window columns' log-sum-exps -- one launch, not two.
+template <typename T>
+__global__ __launch_bounds__(256) void attn_window_merge(RowList rows, int hq, int hkv, AttnWorkspace w,
+                                                         T* __restrict__ out, WindowFuse wf) {
+  const int b = blockIdx.y;
+  if ((int)blockIdx.x < hq) {
+    merge_body<T>(rows, hq, w, out, 1, 0, blockIdx.x, b);
+  } else {
+    const int A = rl_score_len(rows, b);
+    window_lse_merge_body(wf.part, wf.lse, b * hkv + (int)blockIdx.x - hq, (A + w.split_rows - 1) / w.split_rows,
+                          w.max_splits);
+  }
+}
+
 // ------------------------------------------------------------ score finish
 // 256 threads, TPT consecutive tokens each, block `bx` of request `b`.  With own_lse the
 // block works out the per-head score normalisers itself from the splits' partial
@@ -496,9 +511,11 @@ int launch_attention_window(const void* q, const RowList& rows, const okv_kv_lay
     return OKV_ERR_UNSUPPORTED;
   }
   if (lay->dtype == OKV_BF16)
-    hipLaunchKernelGGL((attn_merge<BF16>), dim3(hq, batch), dim3(256), 0, stream, rows, hq, w, (BF16*)out, 1, 0);
+    hipLaunchKernelGGL((attn_window_merge<BF16>), dim3(hq + hkv, batch), dim3(256), 0, stream, rows, hq, hkv, w,
+                       (BF16*)out, wf);
   else
-    hipLaunchKernelGGL((attn_merge<F16>), dim3(hq, batch), dim3(256), 0, stream, rows, hq, w, (F16*)out, 1, 0);
+    hipLaunchKernelGGL((attn_window_merge<F16>), dim3(hq + hkv, batch), dim3(256), 0, stream, rows, hq, hkv, w,
+                       (F16*)out, wf);
   OKV_HIP_CHECK(hipGetLastError());
   return OKV_OK;
 }

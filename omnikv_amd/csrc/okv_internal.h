@@ -189,7 +189,44 @@ struct WindowFuse {
   int64_t q_batch_stride, q_head_stride, q_pos_stride;
   int32_t window;
   float* part;  // [batch][Hkv][kWinCols][max_splits]  log2-domain partial log-sum-exp
+  float* lse;   // [batch][Hkv][kWinCols]  the partials merged (the pass's merge launch does it)
 };
+
+#ifdef __HIPCC__
+// One (request, kv head) of the window columns: the splits' partial log-sum-exps of each of the 64
+// columns folded into one.  256 threads: 64 columns x 4 split lanes, independent loads.
+__device__ __forceinline__ void window_lse_merge_body(const float* __restrict__ part, float* __restrict__ lse,
+                                                      int bg, int num_splits, int max_splits) {
+  __shared__ float sM[4][kWinCols], sD[4][kWinCols];
+  const int c = threadIdx.x & 63, sl = threadIdx.x >> 6;
+  const float* p = part + ((int64_t)bg * kWinCols + c) * max_splits;
+  float M = -INFINITY, den = 0.f;
+  constexpr int U = 8;
+  for (int s0 = sl; s0 < num_splits; s0 += 4 * U) {
+    float x[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) x[u] = s0 + 4 * u < num_splits ? p[s0 + 4 * u] : -INFINITY;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const float mn = fmaxf(M, x[u]);
+      if (mn != -INFINITY) {
+        den = fmaf(den, exp2f(M - mn), exp2f(x[u] - mn));
+        M = mn;
+      }
+    }
+  }
+  sM[sl][c] = M;
+  sD[sl][c] = den;
+  __syncthreads();
+  if (sl == 0) {
+    float Mt = fmaxf(fmaxf(sM[0][c], sM[1][c]), fmaxf(sM[2][c], sM[3][c]));
+    float d = 0.f;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) d += sM[x][c] == -INFINITY ? 0.f : sD[x][c] * exp2f(sM[x][c] - Mt);
+    lse[(int64_t)bg * kWinCols + c] = Mt + log2f(d);
+  }
+}
+#endif
 
 size_t attn_workspace_bytes(int batch, int hq, int hkv, int d, int max_main, int max_tail,
                             int max_score, bool with_v, bool with_logits,

@@ -98,21 +98,24 @@ __global__ __launch_bounds__(256) void window_lse_mfma(WindowArgs a) {
   }
   auto compute = [&](int tbase, const uint4 (&kf)[4]) {
     const int row0 = tbase + 4 * j4;
+    const bool ragged = tbase + 16 > end;  // wave-uniform: only a split's last tile has rows to mask
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) {
       f32x4_t S = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < 4; ++s) S = mfma16((const T*)nullptr, kf[s], qf[cb][s], S);
       float sv[4] = {S[0], S[1], S[2], S[3]};
+      if (ragged) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (row0 + i >= end) sv[i] = -INFINITY;
+        for (int i = 0; i < 4; ++i)
+          if (row0 + i >= end) sv[i] = -INFINITY;
+      }
       const float mn = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), m[cb]);
-      const float ms = mn == -INFINITY ? 0.f : mn;
-      const float alpha = __builtin_amdgcn_exp2f((m[cb] - ms) * sl2);
+      const float ms = (mn == -INFINITY ? 0.f : mn) * sl2;
+      const float alpha = __builtin_amdgcn_exp2f(fmaf(m[cb], sl2, -ms));
       float p = 0.f;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) p += __builtin_amdgcn_exp2f((sv[i] - ms) * sl2);
+      for (int i = 0; i < 4; ++i) p += __builtin_amdgcn_exp2f(fmaf(sv[i], sl2, -ms));
       l[cb] = fmaf(l[cb], alpha, p);
       m[cb] = mn;
     }
@@ -165,50 +168,45 @@ __global__ __launch_bounds__(256) void window_lse_mfma(WindowArgs a) {
   }
 }
 
-// grid (batch * kv heads), 256 threads: 64 columns x 4 split lanes, independent loads
+// grid (batch * kv heads), 256 threads
 __global__ __launch_bounds__(256) void window_lse_merge(WindowArgs a) {
-  __shared__ float sM[4][kWinCols], sD[4][kWinCols];
-  const int bg = blockIdx.x, b = bg / a.hkv, c = threadIdx.x & 63, sl = threadIdx.x >> 6;
-  const int A = win_len(a, b);
-  const int ns = (A + a.split_rows - 1) / a.split_rows;
-  const float* p = a.part + ((int64_t)bg * kWinCols + c) * a.max_splits;
-  float M = -INFINITY, den = 0.f;
-  constexpr int U = 8;
-  for (int s0 = sl; s0 < ns; s0 += 4 * U) {
-    float x[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) x[u] = s0 + 4 * u < ns ? p[s0 + 4 * u] : -INFINITY;
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const float mn = fmaxf(M, x[u]);
-      if (mn != -INFINITY) {
-        den = fmaf(den, exp2f(M - mn), exp2f(x[u] - mn));
-        M = mn;
-      }
-    }
-  }
-  sM[sl][c] = M;
-  sD[sl][c] = den;
-  __syncthreads();
-  if (sl == 0) {
-    float Mt = fmaxf(fmaxf(sM[0][c], sM[1][c]), fmaxf(sM[2][c], sM[3][c]));
-    float d = 0.f;
-#pragma unroll
-    for (int x = 0; x < 4; ++x) d += sM[x][c] == -INFINITY ? 0.f : sD[x][c] * exp2f(sM[x][c] - Mt);
-    a.lse[(int64_t)bg * kWinCols + c] = Mt + log2f(d);
-  }
+  const int bg = blockIdx.x;
+  const int A = win_len(a, bg / a.hkv);
+  window_lse_merge_body(a.part, a.lse, bg, (A + a.split_rows - 1) / a.split_rows, a.max_splits);
 }
 
-// lane i of every quad reads lane perm[i]: 0xB1 = {1,0,3,2} (xor 1), 0x4E = {2,3,0,1} (xor 2)
-template <int QUAD_PERM>
-__device__ __forceinline__ float quad_swap(float x) {
-  return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), QUAD_PERM, 0xf, 0xf, true));
+// Max over the G neighbouring lanes (G = 1, 2, 4 or 8) of four values at once, each step one
+// v_max_f32 with a DPP operand: xor 1 and xor 2 inside the quad, then the mirrored lane of the half
+// row (any lane of the other quad holds that quad's max by then).  The
+// leading s_nop covers the two wait states between a VALU write and a DPP read of the same
+// register; inside the block three other instructions separate every write from its DPP read.
+#define OKV_DPP_MAX4(CTRL)                                                        \
+  "v_max_f32_dpp %0, %0, %0 " CTRL " row_mask:0xf bank_mask:0xf\n\t"              \
+  "v_max_f32_dpp %1, %1, %1 " CTRL " row_mask:0xf bank_mask:0xf\n\t"              \
+  "v_max_f32_dpp %2, %2, %2 " CTRL " row_mask:0xf bank_mask:0xf\n\t"              \
+  "v_max_f32_dpp %3, %3, %3 " CTRL " row_mask:0xf bank_mask:0xf\n\t"
+template <int G>
+__device__ __forceinline__ void group_max4(float& a, float& b, float& c, float& d) {
+  if (G == 2)
+    asm volatile("s_nop 1\n\t" OKV_DPP_MAX4("quad_perm:[1,0,3,2]") : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+  else if (G == 4)
+    asm volatile("s_nop 1\n\t" OKV_DPP_MAX4("quad_perm:[1,0,3,2]") OKV_DPP_MAX4("quad_perm:[2,3,0,1]")
+                 : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+  else if (G == 8)
+    asm volatile("s_nop 1\n\t" OKV_DPP_MAX4("quad_perm:[1,0,3,2]") OKV_DPP_MAX4("quad_perm:[2,3,0,1]")
+                     OKV_DPP_MAX4("row_half_mirror")
+                 : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
 }
+#undef OKV_DPP_MAX4
 
 // ------------------------------------------------------------------ pass 2
-// grid (row blocks, batch), one wave per kv head; LDS: [window][rows_per_block + 1] bit
+// words between two positions' rows in LDS: 16 mod 64, so that the (up to) 4 positions x 16 rows
+// which one atomic instruction touches fall into different banks
+__host__ __device__ inline int window_row_stride(int rows_per_block) { return (rows_per_block + 47) / 64 * 64 + 16; }
+
+// grid (row blocks, batch), one wave per kv head; LDS: [window][window_row_stride] bit
 // patterns of non-negative floats (their unsigned order is their numeric order).
-template <typename T, int NCB>
+template <typename T, int NCB, int G>
 __global__ __launch_bounds__(512, 4) void window_score_mfma(WindowArgs a, int rows_per_block, int exp_decay,
                                                          float* __restrict__ scores,
                                                          int64_t score_stride) {
@@ -220,22 +218,24 @@ __global__ __launch_bounds__(512, 4) void window_score_mfma(WindowArgs a, int ro
   if (begin >= end) return;
   const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
   const int r16 = lane & 15, j4 = lane >> 4;
+  const int nrows = end - begin;
 
-  // rows one word apart per position: the 4 positions x 4 lane rows of one atomic instruction
-  // then fall into 16 different banks (a stride that is a multiple of 32 words puts the
-  // positions on one bank: 74% of the LDS cycles were conflicts)
-  const int wstride = rows_per_block + 1;
+  const int wstride = window_row_stride(rows_per_block);
   for (int i = threadIdx.x; i < a.window * wstride; i += blockDim.x) wmax[i] = 0u;
 
   uint4 qf[NCB][4];
   load_window_q<T, NCB>(a, b, g, r16, j4, qf);
+  // The q heads of a kv head sit in G neighbouring columns.  After the max
+  // over them every lane of the group holds the group's four rows; lane `sub` of the group
+  // reports row `sub`, so one atomic instruction carries min(G, 4) rows of every position.
+  const int sub = r16 & (G - 1);
   float lse[NCB];
-  int wcol[NCB];  // position of this lane's column, or -1 when the lane does not report it
+  int wrow[NCB];  // first word of this lane's position's row of maxima, or -1 when the lane reports nothing
 #pragma unroll
   for (int cb = 0; cb < NCB; ++cb) {
     const int c = 16 * cb + r16;
     lse[cb] = a.lse[(int64_t)(b * a.hkv + g) * kWinCols + c];
-    wcol[cb] = (c % a.group == 0 && c / a.group < a.window) ? c / a.group : -1;
+    wrow[cb] = (sub < 4 && c / G < a.window) ? (c / G) * wstride : -1;
   }
   const T* kb = reinterpret_cast<const T*>(a.k_base) + (int64_t)b * a.batch_stride +
                 (int64_t)g * a.head_stride + 8 * j4;
@@ -249,6 +249,11 @@ __global__ __launch_bounds__(512, 4) void window_score_mfma(WindowArgs a, int ro
     for (int s = 0; s < 4; ++s) kf[s] = *reinterpret_cast<const uint4*>(kp + 32 * s);
   };
   const float sl2 = a.scale * kLog2e;
+  // exp2 is applied after the max over the heads (it is monotonic: the largest exponent gives the
+  // largest probability), once per reported row instead of once per logit
+  auto report = [&](int cb, float x, int row) {
+    if (wrow[cb] >= 0 && row < nrows) atomicMax(&wmax[wrow[cb] + row], __float_as_uint(__builtin_amdgcn_exp2f(x)));
+  };
   auto compute = [&](int tbase, const uint4 (&kf)[4]) {
     const int row0 = tbase + 4 * j4 - begin;
 #pragma unroll
@@ -256,15 +261,19 @@ __global__ __launch_bounds__(512, 4) void window_score_mfma(WindowArgs a, int ro
       f32x4_t S = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < 4; ++s) S = mfma16((const T*)nullptr, kf[s], qf[cb][s], S);
+      float x[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float p = __builtin_amdgcn_exp2f(fmaf(S[i], sl2, -lse[cb]));
-        // max over the q heads of the kv head: neighbours inside a quad by DPP, beyond by a swap
-        if (a.group >= 2) p = fmaxf(p, quad_swap<0xB1>(p));
-        if (a.group >= 4) p = fmaxf(p, quad_swap<0x4E>(p));
-        if (a.group >= 8) p = fmaxf(p, __shfl_xor(p, 4));
-        if (wcol[cb] >= 0 && row0 + i < end - begin)
-          atomicMax(&wmax[wcol[cb] * wstride + row0 + i], __float_as_uint(p));
+      for (int i = 0; i < 4; ++i) x[i] = fmaf(S[i], sl2, -lse[cb]);
+      group_max4<G>(x[0], x[1], x[2], x[3]);
+      if (G >= 4) {
+        const float lo = sub & 1 ? x[1] : x[0], hi = sub & 1 ? x[3] : x[2];
+        report(cb, sub & 2 ? hi : lo, row0 + sub);
+      } else if (G == 2) {
+        report(cb, sub ? x[1] : x[0], row0 + sub);
+        report(cb, sub ? x[3] : x[2], row0 + 2 + sub);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) report(cb, x[i], row0 + i);
       }
     }
   };
@@ -287,7 +296,7 @@ __global__ __launch_bounds__(512, 4) void window_score_mfma(WindowArgs a, int ro
     }
   }
   __syncthreads();
-  for (int r = threadIdx.x; r < end - begin; r += blockDim.x) {
+  for (int r = threadIdx.x; r < nrows; r += blockDim.x) {
     // the reference's order: positions oldest first, running sum (uniform) or
     // running sum halved before each addition (exp)
     float acc = __uint_as_float(wmax[r]);
@@ -324,38 +333,54 @@ size_t window_workspace_bytes(int batch, int hkv, int max_len) {
   return window_part_bytes(batch, hkv, splits);
 }
 
-template <typename T, int NCB>
+template <typename T, int NCB, int G>
 static void launch_window(WindowArgs a, int batch, int exp_decay, float* scores, int64_t score_stride,
-                          int cus, hipStream_t stream, bool lse_parts_ready) {
-  if (!lse_parts_ready)  // otherwise the dense pass of the same call has left them
+                          int cus, hipStream_t stream, bool lse_ready) {
+  if (!lse_ready) {  // otherwise the dense pass of the same call and its merge launch have left them
     hipLaunchKernelGGL((window_lse_mfma<T, NCB>), dim3(a.hkv, a.max_splits, batch), dim3(256), 0, stream, a);
-  hipLaunchKernelGGL(window_lse_merge, dim3(batch * a.hkv), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL(window_lse_merge, dim3(batch * a.hkv), dim3(256), 0, stream, a);
+  }
   // one round of row blocks, two blocks of `hkv` waves per CU; LDS bounds the rows
   int64_t per = ((int64_t)a.max_score_len * batch + 2 * cus - 1) / (2 * cus);
   int rpb = (int)((per + 15) / 16 * 16);
   if (rpb < 64) rpb = 64;
-  const int cap = (48 * 1024 / 4 / a.window) / 16 * 16;
+  const int cap = (48 * 1024 / 4 / a.window - 16) / 64 * 64 + 16;  // window_row_stride(cap) == cap: 48 KB of LDS at most
   if (rpb > cap) {  // several rounds of one block per CU: equal ones
     const int64_t rounds = (per + cap - 1) / cap;
     rpb = (int)(((per + rounds - 1) / rounds + 15) / 16 * 16);
   }
   dim3 grid((a.max_score_len + rpb - 1) / rpb, batch);
-  hipLaunchKernelGGL((window_score_mfma<T, NCB>), grid, dim3(64 * a.hkv),
-                     (size_t)a.window * (rpb + 1) * sizeof(uint32_t), stream, a, rpb, exp_decay, scores,
+  hipLaunchKernelGGL((window_score_mfma<T, NCB, G>), grid, dim3(64 * a.hkv),
+                     (size_t)a.window * window_row_stride(rpb) * sizeof(uint32_t), stream, a, rpb, exp_decay, scores,
                      score_stride);
 }
 
-template <typename T>
-static void launch_window_t(const WindowArgs& a, int batch, int exp_decay, float* scores,
-                            int64_t score_stride, int cus, hipStream_t stream, bool lse_parts_ready = false) {
-  const int ncb = (a.window * a.group + 15) / 16;
+template <typename T, int G>
+static void launch_window_g(const WindowArgs& a, int batch, int exp_decay, float* scores, int64_t score_stride,
+                            int cus, hipStream_t stream, bool lse_ready) {
+  const int ncb = (a.window * G + 15) / 16;
   switch (ncb) {
-    case 1: launch_window<T, 1>(a, batch, exp_decay, scores, score_stride, cus, stream, lse_parts_ready); break;
-    case 2: launch_window<T, 2>(a, batch, exp_decay, scores, score_stride, cus, stream, lse_parts_ready); break;
-    case 3: launch_window<T, 3>(a, batch, exp_decay, scores, score_stride, cus, stream, lse_parts_ready); break;
-    default: launch_window<T, 4>(a, batch, exp_decay, scores, score_stride, cus, stream, lse_parts_ready); break;
+    case 1: launch_window<T, 1, G>(a, batch, exp_decay, scores, score_stride, cus, stream, lse_ready); break;
+    case 2: launch_window<T, 2, G>(a, batch, exp_decay, scores, score_stride, cus, stream, lse_ready); break;
+    case 3: launch_window<T, 3, G>(a, batch, exp_decay, scores, score_stride, cus, stream, lse_ready); break;
+    default: launch_window<T, 4, G>(a, batch, exp_decay, scores, score_stride, cus, stream, lse_ready); break;
   }
 }
+
+// the q heads per kv head: 1, 2, 4 or 8 (window_group_supported)
+template <typename T>
+static void launch_window_t(const WindowArgs& a, int batch, int exp_decay, float* scores,
+                            int64_t score_stride, int cus, hipStream_t stream, bool lse_ready = false) {
+  switch (a.group) {
+    case 1: launch_window_g<T, 1>(a, batch, exp_decay, scores, score_stride, cus, stream, lse_ready); break;
+    case 2: launch_window_g<T, 2>(a, batch, exp_decay, scores, score_stride, cus, stream, lse_ready); break;
+    case 4: launch_window_g<T, 4>(a, batch, exp_decay, scores, score_stride, cus, stream, lse_ready); break;
+    case 8: launch_window_g<T, 8>(a, batch, exp_decay, scores, score_stride, cus, stream, lse_ready); break;
+    default: break;  // refused by the entry points
+  }
+}
+
+static bool window_group_supported(int group) { return group == 1 || group == 2 || group == 4 || group == 8; }
 
 // bytes of the window columns' partials and merged log-sum-exps for `splits` splits per request
 static size_t window_part_bytes(int batch, int hkv, int splits) {
@@ -394,6 +419,8 @@ extern "C" int okv_score_window(const void* q, int64_t q_batch_stride, int64_t q
   OKV_REQUIRE(layout->page_table == nullptr, OKV_ERR_UNSUPPORTED, "window scoring reads contiguous K only");
   OKV_REQUIRE(window * group <= kWinCols, OKV_ERR_UNSUPPORTED,
               "window %d x group %d exceeds %d query rows per kv head", window, group, kWinCols);
+  OKV_REQUIRE(window_group_supported(group), OKV_ERR_UNSUPPORTED,
+              "window scoring takes 1, 2, 4 or 8 q heads per kv head, not %d", group);
   OKV_REQUIRE(hkv <= 8, OKV_ERR_UNSUPPORTED, "more than 8 kv heads");
   OKV_REQUIRE(layout->token_stride < (1ll << 31), OKV_ERR_UNSUPPORTED, "token stride too large");
   if (max_score_len == 0) return OKV_OK;
@@ -451,6 +478,8 @@ extern "C" int okv_dense_attn_window(const void* q, const void* q_window, int64_
   OKV_REQUIRE(layout->page_table == nullptr, OKV_ERR_UNSUPPORTED, "window scoring reads contiguous K only");
   OKV_REQUIRE(window * group <= kWinCols, OKV_ERR_UNSUPPORTED,
               "window %d x group %d exceeds %d query rows per kv head", window, group, kWinCols);
+  OKV_REQUIRE(window_group_supported(group), OKV_ERR_UNSUPPORTED,
+              "window scoring takes 1, 2, 4 or 8 q heads per kv head, not %d", group);
   OKV_REQUIRE(hkv <= 8, OKV_ERR_UNSUPPORTED, "more than 8 kv heads");
   OKV_REQUIRE(layout->token_stride < (1ll << 31), OKV_ERR_UNSUPPORTED, "token stride too large");
   const size_t need = dense_window_workspace_bytes(batch, hq, hkv, layout->head_dim, max_seq_len, max_score_len);
@@ -489,6 +518,7 @@ extern "C" int okv_dense_attn_window(const void* q, const void* q_window, int64_
   wf.q_pos_stride = q_pos_stride;
   wf.window = window;
   wf.part = a.part;
+  wf.lse = a.lse;
   RowList r;
   fill_main(&r, k_base, v_base, layout);
   r.main_lens = seq_lens;

@@ -174,7 +174,9 @@ def window_supported(q: torch.Tensor, k) -> bool:
         return False
     hq, w = q.shape[1], q.shape[2]
     hkv = k.shape[1]
-    return k.dtype == q.dtype and hkv <= 8 and hq % hkv == 0 and w * (hq // hkv) <= 64
+    if k.dtype != q.dtype or hkv > 8 or hq % hkv:
+        return False
+    return hq // hkv in (1, 2, 4, 8) and w * (hq // hkv) <= 64  # the kernel's max over a kv head's q heads pairs lanes
 
 
 def score_window(q, k, score_len: Optional[int] = None, selector: str = "uniform", scale: Optional[float] = None,

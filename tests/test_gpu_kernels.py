@@ -382,7 +382,7 @@ def _window_inputs(n, w, hq, hkv, dtype, seed=3, bsz=1):
 @pytest.mark.parametrize("selector", ["uniform", "exp"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("w,hq,hkv,n", [(1, 32, 8, 1000), (3, 32, 8, 4096), (16, 32, 8, 4099), (16, 32, 8, 70001),
-                                        (8, 32, 4, 3000), (5, 8, 8, 2048), (7, 16, 8, 777)])
+                                        (8, 32, 4, 3000), (5, 8, 8, 2048), (7, 16, 8, 777), (8, 8, 1, 1500)])
 def test_window_scores_match_oracle(selector, dtype, w, hq, hkv, n):
     """All window positions in two passes over K (matrix cores) against the oracle's
     position-by-position loop on the same 16-bit values."""
@@ -487,6 +487,13 @@ def test_window_unsupported_shapes_are_refused():
     assert not ops.window_supported(q32.to(DEV), k32.to(DEV))
     with pytest.raises(Exception, match="unsupported"):
         ops.score_window(q32.to(DEV), k32.to(DEV), selector="uniform")
+    q3, k3 = _window_inputs(256, 4, 24, 8, torch.bfloat16)  # three q heads per kv head: the head max pairs lanes
+    assert not ops.window_supported(q3.to(DEV), k3.to(DEV))
+    with pytest.raises(Exception, match="unsupported"):
+        ops.score_window(q3.to(DEV), k3.to(DEV), selector="uniform")
+    v3 = torch.zeros_like(k3)
+    with pytest.raises(Exception, match="unsupported"):
+        ops.dense_attn_window(q3.to(DEV)[:, :, -1:].contiguous(), q3.to(DEV), k3.to(DEV), v3.to(DEV), selector="uniform")
 
 
 # ------------------------------------------------------------------ other GQA group sizes
