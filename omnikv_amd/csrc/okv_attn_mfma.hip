@@ -503,22 +503,29 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
   // ---- a scored split hands its logits over, then LDS changes hands
   if (scored) {
     __syncthreads();
-    const int quads = w.split_rows >> 2;
+    const int quads = (end - begin + 3) >> 2;
     const int nh = w.group_reduce ? 1 : G;  // logits rows this kv head contributes
-    for (int o = threadIdx.x; o < nh * quads; o += 256) {
-      const int h = o / quads, r = begin + 4 * (o % quads);
-      if (r >= end) continue;
-      const float4 v = *reinterpret_cast<const float4*>(slog + h * w.split_rows + (r - begin));
-      float* lp = w.logits + (int64_t)(b * w.logit_heads + g * nh + h) * w.logits_stride + r;
-      if (r + 3 < end) {
-        *reinterpret_cast<float4*>(lp) = v;
-      } else {
-        lp[0] = v.x;
-        if (r + 1 < end) lp[1] = v.y;
-        if (r + 2 < end) lp[2] = v.z;
+    for (int h = 0; h < nh; ++h) {
+      float* lrow = w.logits + (int64_t)(b * w.logit_heads + g * nh + h) * w.logits_stride + begin;
+      const float* srow = slog + h * w.split_rows;
+#pragma unroll 2
+      for (int qd = threadIdx.x; qd < quads; qd += 256) {
+        const int rr = 4 * qd;
+        const float4 v = *reinterpret_cast<const float4*>(srow + rr);
+        if (begin + rr + 3 < end) {
+          *reinterpret_cast<float4*>(lrow + rr) = v;
+        } else {
+          lrow[rr] = v.x;
+          if (begin + rr + 1 < end) lrow[rr + 1] = v.y;
+          if (begin + rr + 2 < end) lrow[rr + 2] = v.z;
+        }
       }
     }
-    __syncthreads();
+    // LDS changes hands once every thread has READ its logits; the stores themselves carry registers
+    // and need not have landed, so the block meets over LDS only
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
   }
 
   // ---- the four waves of the block meet in LDS
@@ -551,7 +558,9 @@ __device__ __forceinline__ void stage1_mfma_body(const T* __restrict__ q, const 
       }
     }
   }
-  __syncthreads();
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");  // over LDS only: the logits' stores may still be on their way
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
   if (WINDOW) {
     if (wscored && threadIdx.x < kWinCols) {
       const int c = threadIdx.x;
