@@ -200,9 +200,9 @@ __device__ __forceinline__ void group_max4(float& a, float& b, float& c, float& 
 #undef OKV_DPP_MAX4
 
 // ------------------------------------------------------------------ pass 2
-// words between two positions' rows in LDS: 16 mod 64, so that the (up to) 4 positions x 16 rows
-// which one atomic instruction touches fall into different banks
-__host__ __device__ inline int window_row_stride(int rows_per_block) { return (rows_per_block + 47) / 64 * 64 + 16; }
+// words between two positions' rows in LDS: 8 mod 32, so that the 4 positions x 8 rows which half a
+// wave's lanes touch in one atomic instruction fall into the 32 different banks
+__host__ __device__ inline int window_row_stride(int rows_per_block) { return (rows_per_block + 23) / 32 * 32 + 8; }
 
 // grid (row blocks, batch), one wave per kv head; LDS: [window][window_row_stride] bit
 // patterns of non-negative floats (their unsigned order is their numeric order).
@@ -344,7 +344,7 @@ static void launch_window(WindowArgs a, int batch, int exp_decay, float* scores,
   int64_t per = ((int64_t)a.max_score_len * batch + 2 * cus - 1) / (2 * cus);
   int rpb = (int)((per + 15) / 16 * 16);
   if (rpb < 64) rpb = 64;
-  const int cap = (48 * 1024 / 4 / a.window - 16) / 64 * 64 + 16;  // window_row_stride(cap) == cap: 48 KB of LDS at most
+  const int cap = (48 * 1024 / 4 / a.window - 8) / 32 * 32;  // window_row_stride(cap) == cap + 8: 48 KB of LDS at most
   if (rpb > cap) {  // several rounds of one block per CU: equal ones
     const int64_t rounds = (per + cap - 1) / cap;
     rpb = (int)(((per + rounds - 1) / rounds + 15) / 16 * 16);
