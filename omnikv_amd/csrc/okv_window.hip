@@ -6,10 +6,10 @@
 //
 //   pass 1  window_lse_mfma    per (position, head): log-sum-exp of its logits over the
 //                              tokens, split-context partials + a small merge
-//   pass 2  window_score_mfma  logits again, probabilities exp(logit - lse), max over the
-//                              heads (lane swaps inside a kv head, LDS atomics across kv
-//                              heads), then the sum over the positions in the
-//                              reference's order of additions
+//   pass 2  window_score_mfma  logits again, max over the q heads of a kv head of
+//                              logit - lse (DPP), one exponential per position and row,
+//                              max over the kv heads by LDS atomics, then the sum over
+//                              the positions in the reference's order of additions
 //
 // The B operand of a kv head g holds its W*G query rows as columns: column c is
 // position c/G, q head g*G + c%G; up to four 16-column blocks (W*G <= 64).
@@ -177,7 +177,8 @@ __global__ __launch_bounds__(256) void window_lse_merge(WindowArgs a) {
 
 // Max over the G neighbouring lanes (G = 1, 2, 4 or 8) of four values at once, each step one
 // v_max_f32 with a DPP operand: xor 1 and xor 2 inside the quad, then the mirrored lane of the half
-// row (any lane of the other quad holds that quad's max by then).  The
+// row (any lane of the other quad holds that quad's max by then).  Written out because fmaxf() on
+// a DPP-moved value makes the compiler quiet every operand with a v_max x, x of its own.  The
 // leading s_nop covers the two wait states between a VALU write and a DPP read of the same
 // register; inside the block three other instructions separate every write from its DPP read.
 #define OKV_DPP_MAX4(CTRL)                                                        \
@@ -279,9 +280,10 @@ __global__ __launch_bounds__(512, 4) void window_score_mfma(WindowArgs a, int ro
   };
   __syncthreads();  // the zero fill is complete
   {
-    // two tiles in flight per wave and 128 registers at most, so that two workgroups fit a CU
-    // (four waves per SIMD: 58 us at 128K against 66 us for one workgroup with four tiles in
-    // flight); every load is unconditional, past the end it repeats the last tile
+    // two tiles in flight per wave, two workgroups per CU (four waves per SIMD): one workgroup
+    // with four tiles in flight is slower, and so are three or four workgroups of shorter row
+    // blocks (every wave first loads its kv head's query fragments); every load is
+    // unconditional, past the end it repeats the last tile
     uint4 kf[2][4];
     const int t_last = begin + ((last - begin) >> 4 << 4);
 #pragma unroll
