@@ -142,7 +142,7 @@ int okv_score(const void* q, const void* k_base, const okv_kv_layout_t* layout,
  * i.e. the additions in the order of the loops they replace:
  * select_tokens_by_attn_universal, branches `uniform` and `exp`,
  * modeling/omnikv.py:59-103.  K is read twice in total, not `window` times.
- * 16-bit contiguous K, at most 8 kv heads, window * group <= 64; anything else
+ * 16-bit contiguous K, at most 8 kv heads, group of 1, 2, 4 or 8, window * group <= 64; anything else
  * returns OKV_ERR_UNSUPPORTED (callers then score position by position with
  * okv_score).  Workspace: okv_workspace_bytes(OKV_OP_SCORE_WINDOW, ...).
  */
