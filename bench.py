@@ -17,7 +17,9 @@ filter layer composes the selected tokens' pool slots once (PagedKV.slot_index) 
 through them.  Same JSON shape for all.
 
 Prints ONE JSON line: metric = microseconds of attention per layer (step time /
-32); `roofline` for the dominant kernel (dense split attention); `roofline_by_kernel`
+32); `roofline` for the dominant kernel (dense split attention), its `traffic` read from the
+hardware's byte counters in two short child runs of rocprofv3 after the timed region
+(`--no-live-traffic` to skip them); `roofline_by_kernel`
 for every kernel of the step (scoring, filter pass, sparse gather-attention, top-k, and
 the load-only floor of the sparse layer), each timed live with events around a replayed
 graph of that kernel alone; `variants` (the reference's `last` selector; k = round
@@ -39,8 +41,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the dense split pass from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE
-# (profiles/dense_split_pass_pmc.txt), keyed by (context, tail, dtype); None when not measured.
+# HBM bytes per launch of the dense split pass from an earlier rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE run
+# (profiles/dense_split_pass_pmc.txt), keyed by (context, tail, dtype): what the line carries when the live
+# measurement (live_traffic) cannot run.
 TRAFFIC_BYTES = {(131072, 1, "bf16"): 537.1e6 + 1.04e6, (450000, 1, "bf16"): 1843.4e6 + 2.11e6}
 HQ, HKV, D, LAYERS = 32, 8, 128, 32
 FILTER_LAYERS = (2, 8, 18)
@@ -139,6 +142,78 @@ def make_step(ks, vs, qs, n, tail, k_sel, selector, overlap_select=False):
         return outs, idx
 
     return step
+
+
+def traffic_from_counters(path, counter, copy_bytes):
+    """One rocprofv3 counter_collection CSV -> bytes per launch of the dense split pass: the average reading over its
+    dispatches (the attention pass itself -- with V, contiguous rows, no logits -- not the scoring pass of the
+    set-up), scaled by the reading of the run's last three dispatches of the runtime's copy kernel, which moved
+    `copy_bytes` each way.  (dict, "") or (None, reason)."""
+    import csv
+
+    dense, copy = [], []  # in dispatch order
+    for r in csv.DictReader(open(path)):
+        if r["Counter_Name"] != counter:
+            continue
+        name = r["Kernel_Name"]
+        if ("attn_stage1_mfma" in name and ", true, 0, false>" in name) or \
+                ("attn_stage1_generic" in name and ", true>" in name):
+            dense.append(float(r["Counter_Value"]))
+        elif "copyBuffer" in name:
+            copy.append(float(r["Counter_Value"]))
+    copy = copy[-3:]
+    if len(dense) < 4 or len(copy) < 3 or min(copy) <= 0:
+        return None, f"{len(dense)} dense and {len(copy)} copy dispatches"
+    raw_dense, raw_copy = sum(dense) / len(dense) * 1024.0, sum(copy) / len(copy) * 1024.0  # the counters count KiB
+    return {"raw_bytes": raw_dense, "scale": copy_bytes / raw_copy, "bytes": raw_dense * copy_bytes / raw_copy,
+            "dispatches": len(dense)}, ""
+
+
+def live_traffic(n, tail, dtype, budget_s=150.0):
+    """HBM bytes per launch of the dense split pass by the hardware's counters, taken now: two child runs of
+    `rocprofv3 --pmc` (FETCH_SIZE, then WRITE_SIZE; one counter per run) around
+    `python -m omnikv_amd.microbench --op dense --then-copy 3` at this shape.  Each counter is scaled by what it
+    reads, in the same process, for the runtime's copy kernel moving one K tensor (a transfer of known size).
+    Returns (dict | None, note): None with the reason when the profiler is absent, fails or runs out of time."""
+    import shutil
+    import signal
+    import subprocess
+    import tempfile
+
+    exe = shutil.which("rocprofv3")
+    if exe is None:
+        return None, "rocprofv3 is not on PATH"
+    if "rocprofiler" in os.environ.get("LD_PRELOAD", ""):
+        return None, "this run is itself being profiled"
+    env = dict(os.environ, TMPDIR="/tmp", PYTHONPATH=ROOT + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    got = {}
+    with tempfile.TemporaryDirectory(dir="/tmp") as td:
+        for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+            out_dir = os.path.join(td, counter)
+            cmd = [exe, "--pmc", counter, "--kernel-trace", "--output-format", "csv", "-d", out_dir, "-o", "p", "--",
+                   sys.executable, "-m", "omnikv_amd.microbench", "--op", "dense", "--ctx", str(n), "--tail", str(tail),
+                   "--dtype", dtype, "--layers", "2", "--reps", "4", "--warmup", "1", "--then-copy", "3"]
+            with open(os.path.join(td, counter + ".log"), "w") as log:
+                child = subprocess.Popen(cmd, cwd="/tmp", env=env, stdout=log, stderr=log, start_new_session=True)
+                try:
+                    rc = child.wait(timeout=budget_s / 2)
+                except subprocess.TimeoutExpired:
+                    os.killpg(child.pid, signal.SIGKILL)  # the group this call started, nothing else
+                    child.wait()
+                    return None, f"the {counter} run did not finish in {budget_s / 2:.0f} s"
+            if rc != 0:
+                return None, f"the {counter} run ended with status {rc}"
+            copy_bytes = None
+            for line in open(os.path.join(td, counter + ".log")):
+                if line.startswith("{"):
+                    copy_bytes = json.loads(line).get("copy_bytes_each_way")
+            path = os.path.join(out_dir, "p_counter_collection.csv")
+            if copy_bytes is None or not os.path.exists(path):
+                return None, f"the {counter} run left no counters"
+            got[counter], why = traffic_from_counters(path, counter, copy_bytes)
+            if got[counter] is None:
+                return None, f"the {counter} run: {why}"
+    return got, "measured in this run"
 
 
 def cpu_baseline(n, k_sel, selector, budget_s=25.0):
@@ -670,6 +745,8 @@ def main():
     ap.add_argument("--overlap-select", action="store_true",
                     help="run each filter layer's top-k on a stream of its own under the wait-load layer (measured slower)")
     ap.add_argument("--no-variants", action="store_true", help="skip the extra steps (selector last, k = round(ratio N))")
+    ap.add_argument("--no-live-traffic", action="store_true",
+                    help="do not re-measure roofline.traffic with rocprofv3 --pmc in child processes (two short runs)")
     ap.add_argument("--split-rows", type=int, default=0, help="override rows per split (0 = automatic)")
     ap.add_argument("--attn-variant", type=int, default=0, help="1 = portable VALU stage 1 for every dtype")
     args = ap.parse_args()
@@ -781,6 +858,21 @@ def main():
         else:
             step_bytes += 2.0 * (k_sel + tail) * HKV * D * esize + 4.0 * k_sel
     traffic = TRAFFIC_BYTES.get((n, tail, args.dtype))
+    traffic_source = ("profiles/dense_split_pass_pmc.txt (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of an earlier run of this "
+                      "kernel at this shape; not measured in this run)") if traffic else None
+    traffic_detail = None
+    if not args.no_live_traffic and args.layout == "hf":
+        live, note = live_traffic(n, tail, args.dtype)
+        if live is not None:
+            traffic = live["FETCH_SIZE"]["bytes"] + live["WRITE_SIZE"]["bytes"]
+            traffic_source = ("live: rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, in two child processes of this run around "
+                              "`python -m omnikv_amd.microbench --op dense --then-copy 3` at this shape; each counter scaled by "
+                              "its reading for the runtime's copy kernel moving one K tensor in the same process")
+            traffic_detail = {"fetched_bytes": live["FETCH_SIZE"]["bytes"], "written_bytes": live["WRITE_SIZE"]["bytes"],
+                              "fetch_scale": live["FETCH_SIZE"]["scale"], "write_scale": live["WRITE_SIZE"]["scale"],
+                              "dispatches": live["FETCH_SIZE"]["dispatches"]}
+        elif traffic_source:
+            traffic_source += f"; the live measurement was skipped: {note}"
     res = {
         "metric": "omnikv_decode_step_attn_us_per_layer",
         "value": wall_ms * 1e3 / LAYERS,
@@ -809,9 +901,7 @@ def main():
         "roofline": {
             "kernel": dom["kernel"],
             "bound": "hbm", "achieved": dom["achieved"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": dom["frac"], "traffic": traffic,
-            "traffic_source": "profiles/dense_split_pass_pmc.txt (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of an earlier "
-                              "run of this kernel at this shape; not measured in this run)" if traffic else None,
+            "frac": dom["frac"], "traffic": traffic, "traffic_source": traffic_source, "traffic_detail": traffic_detail,
             "bytes_per_launch": dense_bytes, "avg_launch_us": split_us,
             "with_merge_launch_us": dense_us,
         },

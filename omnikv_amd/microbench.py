@@ -53,6 +53,9 @@ def main():
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32"])
     ap.add_argument("--split-rows", type=int, default=0)
     ap.add_argument("--attn-variant", type=int, default=0)
+    ap.add_argument("--then-copy", type=int, default=0,
+                    help="after the op, copy one K tensor this many times with the runtime's copy kernel: a transfer of "
+                         "known size in the same process, against which hardware byte counters are scaled")
     args = ap.parse_args()
 
     from . import _lib as okv_lib
@@ -236,6 +239,12 @@ def main():
         if args.op == "offload_incremental":
             res.update({"overlap": args.overlap, "rows_fetched_per_layer": off.last_fetch_count(0),
                         "full_restage_bytes": 2.0 * k_sel * row * nl})
+    if args.then_copy > 0:
+        cdst = torch.empty_like(ks[0])
+        for _ in range(args.then_copy):
+            cdst.copy_(ks[0])
+        torch.cuda.synchronize()
+        res["copy_bytes_each_way"] = ks[0].numel() * es
     print(json.dumps(res))
 
 

@@ -372,3 +372,28 @@ def test_llama_checkpoint_names_load_into_the_merged_projections():
     sd["model.layers.1.mlp.up_proj.weight"] = torch.zeros(3, 3)
     with pytest.raises(ValueError, match="shape"):
         lm.load_llama_state_dict(sd)
+
+
+def test_bench_scales_the_byte_counters_by_the_copy_kernel(tmp_path, monkeypatch):
+    """bench.py's live roofline.traffic: the dense pass's average counter reading, scaled by what the same counter
+    reads for the copy kernel's known transfer; the set-up's scoring pass and earlier copies are left out; without a
+    profiler the measurement is skipped with a reason."""
+    import bench
+
+    head = '"Dispatch_Id","Kernel_Name","Grid_Size","Counter_Name","Counter_Value"\n'
+    dense = "void okv::attn_stage1_mfma<okv::BF16, 4, true, 0, false>(okv::BF16 const*, okv::RowList, int, float, okv::AttnWorkspace)"
+    score = "void okv::attn_stage1_mfma<okv::BF16, 4, false, 0, true>(okv::BF16 const*, okv::RowList, int, float, okv::AttnWorkspace)"
+    rows = [(1, "__amd_rocclr_copyBuffer", 77.0), (2, score, 999999.0)]
+    rows += [(3 + i, dense, 262256.0) for i in range(5)]
+    rows += [(8 + i, "__amd_rocclr_copyBuffer", 131089.0) for i in range(3)]
+    path = tmp_path / "p_counter_collection.csv"
+    path.write_text(head + "".join(f'{d},"{k}",1024,"FETCH_SIZE",{v}\n' for d, k, v in rows)
+                    + '20,"' + dense + '",1024,"WRITE_SIZE",5.0\n')
+    got, why = bench.traffic_from_counters(str(path), "FETCH_SIZE", 268437504)
+    assert why == "" and got["dispatches"] == 5
+    assert abs(got["scale"] - 268437504 / (131089.0 * 1024)) < 1e-12
+    assert abs(got["bytes"] - 262256.0 * 1024 * got["scale"]) < 1.0
+    none, why = bench.traffic_from_counters(str(path), "WRITE_SIZE", 268437504)
+    assert none is None and "1 dense" in why
+    monkeypatch.setattr("shutil.which", lambda name: None)
+    assert bench.live_traffic(131072, 1, "bf16") == (None, "rocprofv3 is not on PATH")
