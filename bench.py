@@ -144,10 +144,10 @@ def make_step(ks, vs, qs, n, tail, k_sel, selector, overlap_select=False):
     return step
 
 
-def traffic_from_counters(path, counter, copy_bytes):
+def traffic_from_counters(path, counter, copy_bytes, mode=0):
     """One rocprofv3 counter_collection CSV -> bytes per launch of the dense split pass: the average reading over its
-    dispatches (the attention pass itself -- with V, contiguous rows, no logits -- not the scoring pass of the
-    set-up), scaled by the reading of the run's last three dispatches of the runtime's copy kernel, which moved
+    dispatches (the attention pass itself -- with V, row mode `mode` (0 contiguous, 3 paged), no logits -- not the
+    scoring pass of the set-up), scaled by the reading of the run's last three dispatches of the runtime's copy kernel, which moved
     `copy_bytes` each way.  (dict, "") or (None, reason)."""
     import csv
 
@@ -156,7 +156,7 @@ def traffic_from_counters(path, counter, copy_bytes):
         if r["Counter_Name"] != counter:
             continue
         name = r["Kernel_Name"]
-        if ("attn_stage1_mfma" in name and ", true, 0, false>" in name) or \
+        if ("attn_stage1_mfma" in name and f", true, {mode}, false>" in name) or \
                 ("attn_stage1_generic" in name and ", true>" in name):
             dense.append(float(r["Counter_Value"]))
         elif "copyBuffer" in name:
@@ -169,10 +169,11 @@ def traffic_from_counters(path, counter, copy_bytes):
             "dispatches": len(dense)}, ""
 
 
-def live_traffic(n, tail, dtype, budget_s=150.0):
+def live_traffic(n, tail, dtype, budget_s=150.0, paged=False):
     """HBM bytes per launch of the dense split pass by the hardware's counters, taken now: two child runs of
     `rocprofv3 --pmc` (FETCH_SIZE, then WRITE_SIZE; one counter per run) around
-    `python -m omnikv_amd.microbench --op dense --then-copy 3` at this shape.  Each counter is scaled by what it
+    `python -m omnikv_amd.microbench --op dense --then-copy 3` at this shape (`--op paged_dense` for the paged
+    batch: the same requests and pool, without the decode step's own token).  Each counter is scaled by what it
     reads, in the same process, for the runtime's copy kernel moving one K tensor (a transfer of known size).
     Returns (dict | None, note): None with the reason when the profiler is absent, fails or runs out of time."""
     import shutil
@@ -191,8 +192,9 @@ def live_traffic(n, tail, dtype, budget_s=150.0):
         for counter in ("FETCH_SIZE", "WRITE_SIZE"):
             out_dir = os.path.join(td, counter)
             cmd = [exe, "--pmc", counter, "--kernel-trace", "--output-format", "csv", "-d", out_dir, "-o", "p", "--",
-                   sys.executable, "-m", "omnikv_amd.microbench", "--op", "dense", "--ctx", str(n), "--tail", str(tail),
-                   "--dtype", dtype, "--layers", "2", "--reps", "4", "--warmup", "1", "--then-copy", "3"]
+                   sys.executable, "-m", "omnikv_amd.microbench", "--dtype", dtype, "--layers", "2", "--reps", "4",
+                   "--warmup", "1", "--then-copy", "3"]
+            cmd += ["--op", "paged_dense"] if paged else ["--op", "dense", "--ctx", str(n), "--tail", str(tail)]
             with open(os.path.join(td, counter + ".log"), "w") as log:
                 child = subprocess.Popen(cmd, cwd="/tmp", env=env, stdout=log, stderr=log, start_new_session=True)
                 try:
@@ -210,7 +212,7 @@ def live_traffic(n, tail, dtype, budget_s=150.0):
             path = os.path.join(out_dir, "p_counter_collection.csv")
             if copy_bytes is None or not os.path.exists(path):
                 return None, f"the {counter} run left no counters"
-            got[counter], why = traffic_from_counters(path, counter, copy_bytes)
+            got[counter], why = traffic_from_counters(path, counter, copy_bytes, 3 if paged else 0)
             if got[counter] is None:
                 return None, f"the {counter} run: {why}"
     return got, "measured in this run"
@@ -663,6 +665,20 @@ def main_batch16_paged(args):
     def pct(p):
         return per_step[min(len(per_step) - 1, int(p * len(per_step)))]
 
+    traffic, traffic_source, traffic_detail = None, None, None
+    if not args.no_live_traffic and args.dtype != "f32":
+        live, note = live_traffic(0, 0, args.dtype, paged=True)
+        if live is not None:
+            traffic = live["FETCH_SIZE"]["bytes"] + live["WRITE_SIZE"]["bytes"]
+            traffic_source = ("live: rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, in two child processes of this run around "
+                              "`python -m omnikv_amd.microbench --op paged_dense --then-copy 3` (the same requests, pages "
+                              "and page table, without the decode step's own token: 16 rows fewer); each counter scaled by "
+                              "its reading for the runtime's copy kernel moving one layer's K pool in the same process")
+            traffic_detail = {"fetched_bytes": live["FETCH_SIZE"]["bytes"], "written_bytes": live["WRITE_SIZE"]["bytes"],
+                              "fetch_scale": live["FETCH_SIZE"]["scale"], "write_scale": live["WRITE_SIZE"]["scale"],
+                              "dispatches": live["FETCH_SIZE"]["dispatches"]}
+        else:
+            traffic_source = f"not measured: {note}"
     res = {
         "metric": "omnikv_decode_step_attn_us_per_layer", "value": wall_ms * 1e3 / LAYERS, "unit": "us/layer", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall_ms, "higher_is_better": False, "scaling": "weak",
@@ -679,7 +695,8 @@ def main_batch16_paged(args):
         "step_hbm_gbs": step_bytes / (wall_ms * 1e-3) / 1e9,
         "step_ms_p10_p50_p90": [round(pct(0.1), 4), round(pct(0.5), 4), round(pct(0.9), 4)],
         "roofline": {"kernel": dom["kernel"], "bound": "hbm", "achieved": dom["achieved"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": dom["frac"], "traffic": None, "traffic_source": None, "bytes_per_launch": dense_bytes,
+                     "frac": dom["frac"], "traffic": traffic, "traffic_source": traffic_source,
+                     "traffic_detail": traffic_detail, "bytes_per_launch": dense_bytes,
                      "avg_launch_us": dom["us"], "with_merge_launch_us": by["dense_attention_op"]["us"]},
         "roofline_by_kernel": by,
         "variants": {},

@@ -374,9 +374,17 @@ def paged(args, dev):
     e1.record(stream)
     e1.synchronize()
     us = e0.elapsed_time(e1) * 1e3 / args.reps
-    print(json.dumps({"op": args.op, "batch": args.batch, "page_size": args.page_size, "tokens": tokens,
-                      "selected": sel, "dtype": args.dtype, "us_per_call": us, "algorithmic_bytes": algo,
-                      "algorithmic_GBps": algo / us / 1e3, "frac_of_8TBps": algo / us / 1e3 / 8000.0}))
+    res = {"op": args.op, "batch": args.batch, "page_size": args.page_size, "tokens": tokens,
+           "selected": sel, "dtype": args.dtype, "us_per_call": us, "algorithmic_bytes": algo,
+           "algorithmic_GBps": algo / us / 1e3, "frac_of_8TBps": algo / us / 1e3 / 8000.0}
+    if args.then_copy > 0:
+        csrc = pools[0].pool_k
+        cdst = torch.empty_like(csrc)
+        for _ in range(args.then_copy):
+            cdst.copy_(csrc)
+        torch.cuda.synchronize()
+        res["copy_bytes_each_way"] = csrc.numel() * es
+    print(json.dumps(res))
 
 
 if __name__ == "__main__":
